@@ -7,7 +7,7 @@ Mixtral 8x7B, plus tiny variants for CPU tests and smoke().
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Optional
+from typing import Optional  # noqa: F401
 
 
 @dataclass
@@ -41,6 +41,172 @@ class ModelConfig:
     def kv_bytes_per_token(self) -> int:
         # bf16 K + V per layer
         return 2 * self.num_kv_heads * self.head_dim * 2 * self.num_layers
+
+
+# ---------------------------------------------------------------------------
+# Fedatar: a per-layer hybrid decoder.  Every layer names its own mixer
+# (a minGRU recurrence or windowed latent attention) and its own
+# feed-forward (dense xIELU, relu^2 mixture of experts, or none), so the
+# configuration is a LIST of layer specs instead of one set of sizes.
+# ---------------------------------------------------------------------------
+@dataclass
+class RotarySpec:
+    """Interleaved-pair rotary positions: pair i of the first `dims`
+    entries turns by position * base**(-2i/dims)."""
+    base: float = 10000.0
+    dims: int = 0
+
+
+@dataclass
+class MinGRUSpec:
+    width: int = 0
+
+
+@dataclass
+class LatentAttentionSpec:
+    heads: int = 1
+    dim: int = 64              # unrotated q/k entries per head
+    rot_dim: int = 16          # rotated q/k entries per head (shared key)
+    vdim: int = 64             # value entries per head
+    kv_rank: int = 64          # cached latent width
+    q_rank: int = 64           # query latent width
+    scale: float = 0.0         # score multiplier; 0 => (dim+rot_dim)**-0.5
+    window: int = 0            # keys seen per query incl. itself; 0 = all
+    rot: RotarySpec = None
+
+    def __post_init__(self):
+        if self.rot is None:
+            self.rot = RotarySpec(dims=self.rot_dim)
+        if not self.scale:
+            self.scale = float(self.dim + self.rot_dim) ** -0.5
+
+    @property
+    def cache_width(self) -> int:
+        return self.kv_rank + self.rot_dim
+
+
+@dataclass
+class DenseFFSpec:
+    ff: int = 0
+
+
+@dataclass
+class MoEFFSpec:
+    experts: int = 1
+    top: int = 1
+    expert_ff: int = 0
+    shared_ff: int = 0         # 0 => no always-on shared expert
+
+
+@dataclass
+class LayerSpec:
+    type: str                  # "mingru" | "latent_attention"
+    mixer: object              # MinGRUSpec | LatentAttentionSpec
+    mlp: object = None         # DenseFFSpec | MoEFFSpec | None
+
+
+@dataclass
+class FedatarConfig:
+    name: str
+    hidden_size: int
+    vocab_size: int
+    layers: list
+    norm_eps: float = 1e-5
+    max_position: int = 1 << 20     # angles are computed, not tabulated
+    architecture: str = "Fedatar"
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def is_moe(self) -> bool:
+        return any(isinstance(l.mlp, MoEFFSpec) for l in self.layers)
+
+    def kv_bytes_per_token(self, itemsize: int = 2) -> int:
+        """Paged bytes per token: only latent-attention layers page
+        anything (latent + shared rotated key); minGRU layers hold one
+        fixed-size state per sequence slot instead."""
+        return max(itemsize, sum(
+            l.mixer.cache_width * itemsize for l in self.layers
+            if l.type == "latent_attention"))
+
+    @staticmethod
+    def from_dict(cfg: dict, name: str = "fedatar",
+                  shapes: Optional[dict] = None) -> "FedatarConfig":
+        """Parse the design's config.json.  `shapes` (tensor name ->
+        shape, from the checkpoint header) fills sizes that the json
+        leaves to the tensors."""
+        shapes = shapes or {}
+        layers = []
+        for i, l in enumerate(cfg["layers"]):
+            m = l.get("mixer") or {}
+            if l["type"] == "mingru":
+                width = m.get("width")
+                if width is None:
+                    width = shapes[f"l{i}.mix.z"][0]
+                mixer = MinGRUSpec(width=int(width))
+            elif l["type"] == "latent_attention":
+                rot = m.get("rot") or {}
+                rot_dim = int(m["rot_dim"])
+                q_rank = m.get("q_rank")
+                if q_rank is None:
+                    q_rank = shapes[f"l{i}.mix.dq"][0]
+                mixer = LatentAttentionSpec(
+                    heads=int(m["heads"]), dim=int(m["dim"]),
+                    rot_dim=rot_dim, vdim=int(m["vdim"]),
+                    kv_rank=int(m["kv_rank"]), q_rank=int(q_rank),
+                    scale=float(m.get("scale") or 0.0),
+                    window=int((m.get("mask") or {}).get("size") or 0),
+                    rot=RotarySpec(base=float(rot.get("base", 10000.0)),
+                                   dims=int(rot.get("dims", rot_dim))))
+            else:
+                raise ValueError(f"layer {i}: unknown mixer {l['type']!r}")
+            f = l.get("mlp")
+            if f is None:
+                mlp = None
+            elif f["kind"] == "dense":
+                mlp = DenseFFSpec(ff=int(f["ff"]))
+            elif f["kind"] == "moe":
+                sh = f.get("shared") or {}
+                mlp = MoEFFSpec(experts=int(f["router"]["experts"]),
+                                top=int(f["router"]["top"]),
+                                expert_ff=int(f["expert"]["ff"]),
+                                shared_ff=int(sh.get("ff") or 0))
+            else:
+                raise ValueError(f"layer {i}: unknown mlp {f['kind']!r}")
+            layers.append(LayerSpec(type=l["type"], mixer=mixer, mlp=mlp))
+        return FedatarConfig(
+            name=name, hidden_size=int(cfg["width"]),
+            vocab_size=int(cfg["vocab"]), layers=layers,
+            norm_eps=float((cfg.get("norm") or {}).get("eps", 1e-5)))
+
+
+def fedatar_preset(name: str, width: int, vocab: int, pattern: str,
+                   heads: int, dim: int, rot_dim: int, vdim: int,
+                   kv_rank: int, q_rank: int, window: int, ff: int,
+                   experts: int, top: int, expert_ff: int, shared_ff: int,
+                   rot_base: float = 10000.0) -> FedatarConfig:
+    """Layer pattern string: one letter pair per layer — mixer `g`
+    (minGRU) or `a` (latent attention), then feed-forward `d` (dense),
+    `m` (mixture) or `-` (none); e.g. "gd am gm"."""
+    layers = []
+    for tok in pattern.split():
+        if tok[0] == "g":
+            mixer, typ = MinGRUSpec(width=width), "mingru"
+        else:
+            mixer, typ = LatentAttentionSpec(
+                heads=heads, dim=dim, rot_dim=rot_dim, vdim=vdim,
+                kv_rank=kv_rank, q_rank=q_rank, window=window,
+                rot=RotarySpec(base=rot_base, dims=rot_dim)), \
+                "latent_attention"
+        mlp = {"d": DenseFFSpec(ff=ff),
+               "m": MoEFFSpec(experts=experts, top=top,
+                              expert_ff=expert_ff, shared_ff=shared_ff),
+               "-": None}[tok[1]]
+        layers.append(LayerSpec(type=typ, mixer=mixer, mlp=mlp))
+    return FedatarConfig(name=name, hidden_size=width, vocab_size=vocab,
+                         layers=layers)
 
 
 # Architectures from the public model cards (random-init weights — no network).
@@ -166,6 +332,20 @@ MODEL_PRESETS = {
         qkv_bias=True,
         tie_embeddings=True,
     ),
+    # tiny Fedatar for CPU tests / smoke: both mixers, all three
+    # feed-forward kinds
+    "tiny-fedatar": fedatar_preset(
+        "tiny-fedatar", width=128, vocab=512, pattern="gd am gm a-",
+        heads=2, dim=32, rot_dim=8, vdim=32, kv_rank=48, q_rank=40,
+        window=24, ff=192, experts=6, top=2, expert_ff=48, shared_ff=64),
+    # layer-shape benchmark points at Mixtral-8x7B's width (one layer
+    # of each kind is enough to price the kernels; see bench.py)
+    "fedatar-4k": fedatar_preset(
+        "fedatar-4k", width=4096, vocab=32000,
+        pattern="gd am gm am gm am gm am",
+        heads=32, dim=128, rot_dim=64, vdim=128, kv_rank=512,
+        q_rank=1536, window=4096, ff=14336, experts=8, top=2,
+        expert_ff=14336, shared_ff=0, rot_base=1000000.0),
     "tiny-moe": ModelConfig(
         name="tiny-moe",
         hidden_size=512,
@@ -243,6 +423,10 @@ class EngineConfig:
     # *.safetensors); None keeps the seed-derived synthetic init
     # (engine/weights.py — the no-network default)
     weights_path: Optional[str] = None
+    # compute dtype: "bfloat16" (serving default) or "float32" (true
+    # 32-bit everywhere; only architectures whose kernels are typed for
+    # it accept this — see engine/models/registry.py)
+    dtype: str = "bfloat16"
     tensor_parallel_size: int = 1
     seed: int = 0
 
@@ -263,6 +447,19 @@ class EngineConfig:
     def tiny_moe(**kw) -> "EngineConfig":
         defaults = dict(
             model=MODEL_PRESETS["tiny-moe"],
+            num_gpu_blocks=64,
+            max_num_seqs=8,
+            max_batched_tokens=2048,
+            max_model_len=512,
+            use_hip_graphs=False,
+        )
+        defaults.update(kw)
+        return EngineConfig(**defaults)
+
+    @staticmethod
+    def tiny_fedatar(**kw) -> "EngineConfig":
+        defaults = dict(
+            model=MODEL_PRESETS["tiny-fedatar"],
             num_gpu_blocks=64,
             max_num_seqs=8,
             max_batched_tokens=2048,

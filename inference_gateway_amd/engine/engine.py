@@ -123,19 +123,29 @@ class LLMEngine:
         self.device = torch.device(
             device if torch.cuda.is_available() else "cpu")
         _maybe_load_tuned_gemms()
-        self.dtype = torch.bfloat16
-        if self.device.type == "cuda" and cfg.model.head_dim != 128:
+        self.dtype = {"bfloat16": torch.bfloat16,
+                      "float32": torch.float32}[cfg.dtype]
+        if self.dtype == torch.float32:
+            # true 32-bit: no reduced-precision matrix mode
+            torch.backends.cuda.matmul.allow_tf32 = False
+            torch.set_float32_matmul_precision("highest")
+        if (self.device.type == "cuda"
+                and getattr(cfg.model, "head_dim", 128) != 128):
             raise ValueError(
                 f"model head_dim {cfg.model.head_dim} is not supported "
                 "on GPU: the MFMA attention kernels are tiled for "
                 "head_dim=128 (CPU reference path has no such limit)")
-        if cfg.model.is_moe:
-            from .models.mixtral import MixtralForCausalLM
+        from .models.registry import build_model, is_recurrent
 
-            self.model = MixtralForCausalLM(cfg.model, self.device, self.dtype)
-        else:
-            self.model = LlamaForCausalLM(cfg.model, self.device, self.dtype)
+        self.model = build_model(cfg.model, self.device, self.dtype)
         self.model.eval()
+        # sequence-level batch metadata (row -> sequence maps, state
+        # slots) is only assembled for models that read it
+        self._seq_meta = getattr(self.model, "needs_seq_meta", False)
+        if is_recurrent(cfg.model) and cfg.enable_prefix_caching:
+            raise ValueError(
+                "prefix caching cannot serve a model with recurrent "
+                "layers: the state at a shared prefix's end is not kept")
         if cfg.weights_path:
             from .weights import load_weights
 
@@ -173,7 +183,8 @@ class LLMEngine:
         self._gr_version = -1
         self._pending = None   # (seqs, ring, event) of the in-flight decode
         if (self.device.type == "cuda" and cfg.use_hip_graphs
-                and not cfg.enforce_eager):
+                and not cfg.enforce_eager
+                and getattr(self.model, "supports_decode_graph", True)):
             from .graph_runner import DecodeGraphRunner
 
             self.graph_runner = DecodeGraphRunner(
@@ -199,15 +210,18 @@ class LLMEngine:
     def _allocate_kv(self, num_blocks: int):
         from ..parallel.comm import tp_world_size
 
+        from .state import allocate_caches
+
         m = self.cfg.model
-        nkv = max(1, m.num_kv_heads // tp_world_size())
-        shape = (num_blocks, nkv, self.cfg.block_size, m.head_dim)
-        caches = []
-        for _ in range(m.num_layers):
-            k = torch.zeros(shape, dtype=self.dtype, device=self.device)
-            v = torch.zeros(shape, dtype=self.dtype, device=self.device)
-            caches.append((k, v))
-        return caches
+        if hasattr(self.model, "cache_specs"):
+            specs = self.model.cache_specs()
+        else:
+            nkv = max(1, m.num_kv_heads // tp_world_size())
+            specs = [("paged_kv", nkv, m.head_dim)] * m.num_layers
+        # one state slot per schedulable sequence (Sequence.slot)
+        return allocate_caches(specs, num_blocks, self.cfg.block_size,
+                               self.cfg.max_num_seqs, self.dtype,
+                               self.device)
 
     # ---------------- request API ----------------
     def add_request(self, prompt_token_ids: List[int],
@@ -403,6 +417,66 @@ class LLMEngine:
                     gr.init_slot(seq, tok)
         return prev + outputs
 
+    # ---------------- forced-token replay ----------------
+    def open_stream(self, seq_id: Optional[int] = None) -> int:
+        """Register a sequence whose tokens are DICTATED step by step
+        (replay_step) instead of sampled: scoring given text, replaying
+        a recorded schedule.  It holds no slot or pages until its first
+        tokens arrive and never enters the sampling scheduler's queue."""
+        if seq_id is None:
+            seq_id = next(self._seq_counter)
+        self._seqs[seq_id] = Sequence(
+            seq_id=seq_id, prompt_token_ids=[],
+            sampling=SamplingParams(max_new_tokens=0))
+        return seq_id
+
+    def close_stream(self, seq_id: int) -> None:
+        """Give back a replayed sequence's slot and pages."""
+        seq = self._seqs.pop(seq_id)
+        if seq.state != SeqState.FINISHED:
+            self.scheduler.finish(seq, "stop")
+
+    @torch.inference_mode()
+    def replay_step(self, feeds, want) -> torch.Tensor:
+        """One engine step with a dictated batch.  feeds: [(seq_id,
+        [next tokens])] — every listed sequence runs exactly these
+        tokens from the cache and state its earlier steps left, all
+        together in one forward (prompt portions beside single decoded
+        tokens).  want: {seq_id: [indices into its new tokens]}.
+        Returns fp32 logits [n_wanted, vocab] in feeds order (and
+        `want` order within a sequence); nothing is sampled."""
+        plan = []
+        for sid, toks in feeds:
+            seq = self._seqs[sid]
+            seq.prompt_token_ids.extend(int(t) for t in toks)
+            plan.append((seq, len(toks)))
+        batch = self.scheduler.schedule_forced(plan)
+        self.num_steps += 1
+        fb = self._build_forward_batch(batch)
+        hidden = self.model(fb, self.kv_caches)
+        # batch row of each sequence's first new token
+        first, row = {}, 0
+        if batch.is_prefill:
+            for seq, take in zip(batch.seqs, batch.prefill_takes):
+                first[seq.seq_id] = row
+                row += take
+            for seq in batch.decode_seqs or []:
+                first[seq.seq_id] = row
+                row += 1
+        else:
+            for seq in batch.seqs:
+                first[seq.seq_id] = row
+                row += 1
+        for seq, _n in plan:
+            seq.prefilled = seq.num_tokens
+        rows = [first[sid] + int(i) for sid, _t in feeds
+                for i in want.get(sid, [])]
+        if not rows:
+            return torch.empty((0, self.cfg.model.vocab_size),
+                               dtype=torch.float32, device=self.device)
+        idx = torch.tensor(rows, dtype=torch.int64, device=self.device)
+        return self.model.compute_logits(hidden[idx]).float()
+
     def _drain_pending(self) -> List[StepOutput]:
         if self._pending is None:
             return []
@@ -501,6 +575,11 @@ class LLMEngine:
                 fb.block_table = bt.to(dev)
                 fb.prefix_lens = torch.tensor(prefixes, dtype=torch.int32,
                                               device=dev)
+            if self._seq_meta:
+                self._attach_seq_meta(
+                    fb, list(batch.seqs) + list(dseqs or []),
+                    list(seq_lens) + [1] * len(dseqs or []),
+                    prefixes + [s.num_tokens - 1 for s in (dseqs or [])], P)
             return fb
         # decode
         B = len(batch.seqs)
@@ -518,7 +597,7 @@ class LLMEngine:
             slots.append(blk * bs + pos % bs)
             bt[i, : len(s.block_ids)] = torch.tensor(s.block_ids,
                                                      dtype=torch.int32)
-        return ForwardBatch(
+        fb = ForwardBatch(
             token_ids=torch.tensor(token_ids, dtype=torch.int64, device=dev),
             positions=torch.tensor(positions, dtype=torch.int32, device=dev),
             slot_mapping=torch.tensor(slots, dtype=torch.int32, device=dev),
@@ -527,11 +606,38 @@ class LLMEngine:
             ctx_lens=ctx.to(dev),
             last_token_indices=torch.arange(B, dtype=torch.int64, device=dev),
         )
+        if self._seq_meta:
+            self._attach_seq_meta(fb, batch.seqs, [1] * B, positions, 0)
+        return fb
+
+    def _attach_seq_meta(self, fb: ForwardBatch, seqs, rows, starts,
+                         num_chunk_rows: int) -> None:
+        """Sequence-level view of the batch rows: row offsets, first
+        position, state slot and block-table row per sequence, and the
+        row -> sequence map (ForwardBatch.seq_*)."""
+        dev = self.device
+        S = len(seqs)
+        cu = [0]
+        for r in rows:
+            cu.append(cu[-1] + r)
+        maxb = max(len(s.block_ids) for s in seqs)
+        bt = torch.zeros((S, maxb), dtype=torch.int32)
+        for i, s in enumerate(seqs):
+            bt[i, : len(s.block_ids)] = torch.tensor(s.block_ids,
+                                                     dtype=torch.int32)
+        fb.seq_cu = torch.tensor(cu, dtype=torch.int32, device=dev)
+        fb.seq_start = torch.tensor(starts, dtype=torch.int32, device=dev)
+        fb.seq_slots = torch.tensor([s.slot for s in seqs],
+                                    dtype=torch.int32, device=dev)
+        fb.seq_block_table = bt.to(dev)
+        fb.row_seq = torch.repeat_interleave(
+            torch.arange(S, dtype=torch.int32),
+            torch.tensor(rows, dtype=torch.int64)).to(dev)
+        fb.seq_rows = list(rows)
+        fb.num_chunk_rows = num_chunk_rows
 
     def _copy_block(self, src: int, dst: int) -> None:
-        for k, v in self.kv_caches:
-            k[dst].copy_(k[src])
-            v[dst].copy_(v[src])
+        self.kv_caches.copy_block(src, dst)
 
     def _fork_at_prefill(self, parent, row_logits) -> List[StepOutput]:
         """Materialize a group's n-1 branches from the parent's freshly
@@ -579,6 +685,9 @@ class LLMEngine:
             # abort guard) and kill prefix-cache reuse
             child.prefilled = plen
             self.scheduler.adopt(child)
+            # recurrent layers: the branch continues from the parent's
+            # state at the end of the prompt
+            self.kv_caches.copy_slot(parent.slot, child.slot)
             self.num_forks += 1
             if gr is not None:
                 gr.write_block_row(child.slot, child.block_ids)

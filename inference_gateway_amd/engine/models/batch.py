@@ -35,6 +35,19 @@ class ForwardBatch:
     decode_block_table: Optional[torch.Tensor] = None
     decode_ctx_lens: Optional[torch.Tensor] = None
 
+    # SEQUENCE-LEVEL view of the same rows, for layers that carry state
+    # per sequence or attend per row through the paged cache (built only
+    # when the model asks: model.needs_seq_meta).  Sequences are the
+    # prefill portions in order, then the decode rows; S of them.
+    seq_cu: Optional[torch.Tensor] = None          # [S+1] int32 row offsets
+    seq_start: Optional[torch.Tensor] = None       # [S] int32 position of
+                                                   #   each seq's first row
+    seq_slots: Optional[torch.Tensor] = None       # [S] int32 state slots
+    seq_block_table: Optional[torch.Tensor] = None  # [S, max_blocks] int32
+    row_seq: Optional[torch.Tensor] = None         # [T] int32 seq of a row
+    seq_rows: Optional[List[int]] = None           # python row counts
+    num_chunk_rows: int = 0                        # rows in prompt portions
+
     @property
     def is_mixed(self) -> bool:
         return self.decode_ctx_lens is not None

@@ -179,6 +179,9 @@ class Scheduler:
                     seq.block_ids, seq.cached_prefix = \
                         self.bm.allocate_for_prompt(seq.prompt_token_ids)
                     seq.prefilled = seq.cached_prefix
+                    # the slot is taken with the FIRST chunk: layers
+                    # with per-sequence state write it from then on
+                    seq.slot = self._free_slots.pop()
                 remaining = seq.prompt_len - seq.prefilled
                 take = min(take, remaining)
                 if take <= 0:
@@ -188,7 +191,8 @@ class Scheduler:
                     # same round samples its first token (a completed
                     # seq must never sit in waiting with take 0)
                     self.waiting.popleft()
-                    seq.slot = self._free_slots.pop()
+                    if seq.slot is None:
+                        seq.slot = self._free_slots.pop()
                     seq.state = SeqState.RUNNING
                 prefills.append(seq)
                 takes.append(take)
@@ -207,7 +211,8 @@ class Scheduler:
                     self.bm.allocate_for_prompt(seq.prompt_token_ids)
                 seq.prefilled = seq.cached_prefix
             self.waiting.popleft()
-            seq.slot = self._free_slots.pop()
+            if seq.slot is None:
+                seq.slot = self._free_slots.pop()
             seq.state = SeqState.RUNNING
             prefills.append(seq)
             takes.append(seq.prompt_len - seq.prefilled)
@@ -308,6 +313,46 @@ class Scheduler:
                 new_blocks.append(
                     (seq.slot, len(seq.block_ids) - 1, seq.block_ids[-1]))
         return new_blocks
+
+    # ---- externally dictated steps (forced-token replay) --------------
+    def schedule_forced(self, feeds) -> ScheduledBatch:
+        """Build the batch for a step whose composition is GIVEN: feeds
+        is [(seq, n)], each sequence runs exactly its next n tokens
+        (already appended to its prompt).  Admission, slots and pages
+        go through the same pools as schedule(): a sequence is admitted
+        (slot + running set) at its first feed and its pages grow on
+        demand.  A single token past position 0 runs as a decode row,
+        anything else as a prompt portion, all in one batch.  Raises
+        RuntimeError when slots or pages run out — the caller dictated
+        an unschedulable step; nothing is preempted."""
+        chunks: List[Sequence] = []
+        takes: List[int] = []
+        decodes: List[Sequence] = []
+        for seq, n in feeds:
+            if seq.state == SeqState.FINISHED or n <= 0:
+                raise ValueError(f"seq {seq.seq_id}: nothing to run")
+            if seq.prefilled + n != seq.num_tokens:
+                raise ValueError(
+                    f"seq {seq.seq_id}: {n} tokens fed but "
+                    f"{seq.num_tokens - seq.prefilled} are pending")
+            if seq.state == SeqState.WAITING:
+                if not self._free_slots:
+                    raise RuntimeError("out of sequence slots")
+                seq.slot = self._free_slots.pop()
+                seq.state = SeqState.RUNNING
+                self.running.append(seq)
+                self.membership_version += 1
+            self.bm.ensure_capacity(seq.block_ids, seq.num_tokens)
+            if n == 1 and seq.prefilled > 0:
+                decodes.append(seq)
+            else:
+                chunks.append(seq)
+                takes.append(n)
+        if not chunks:
+            return ScheduledBatch(is_prefill=False, seqs=decodes)
+        return ScheduledBatch(is_prefill=True, seqs=chunks,
+                              prefill_takes=takes,
+                              decode_seqs=decodes or None)
 
     # ---- forked sequences (OpenAI n>1: one prefill, shared prompt KV) --
     def can_adopt(self) -> bool:

@@ -256,6 +256,85 @@ def load_mixtral_weights(model, path: str) -> int:
     return loaded
 
 
+def load_fedatar_weights(model, path: str) -> int:
+    """Load a Fedatar checkpoint: tensors `l<i>.norm1|norm2[.b]`,
+    `l<i>.mix.*`, `l<i>.mlp.*`, `embed`, `final.norm[.b]`, `head`.  The
+    engine's fused layouts are assembled here: z|x|g stacked for the
+    minGRU input GEMM; query-latent | kv-latent+rotated-key | head-gate
+    stacked for the attention down projection; per-head key/value
+    up-projections reshaped for the absorbed batched GEMMs; experts
+    stacked K-major.  Norm weights, sinks, activation constants and the
+    router stay fp32."""
+    from .config import DenseFFSpec, MoEFFSpec
+
+    sh = _Shards(path)
+    cfg = model.cfg
+    n = 0
+
+    def put(param, src, what):
+        nonlocal n
+        _copy(param, src, what)
+        n += 1
+
+    def norm(params, name):
+        put(params.weight, sh.full(name), name)
+        put(params.bias, sh.full(name + ".b"), name + ".b")
+
+    put(model.embed, sh.full("embed"), "embed")
+    for i, (spec, layer) in enumerate(zip(cfg.layers, model.layers)):
+        p = f"l{i}."
+        norm(layer.norm1, p + "norm1")
+        mx, m = layer.mixer, p + "mix."
+        if spec.type == "mingru":
+            W = spec.mixer.width
+            put(mx.zxg, torch.cat([sh.full(m + "z"), sh.full(m + "x"),
+                                   sh.full(m + "g")], 0), m + "z|x|g")
+            put(mx.zxg_b, torch.cat([
+                sh.full(m + "z.b"), sh.full(m + "x.b"),
+                torch.zeros(W, dtype=sh.full(m + "z.b").dtype)], 0),
+                m + "z.b|x.b")
+            put(mx.o, sh.full(m + "o"), m + "o")
+        else:
+            a = spec.mixer
+            put(mx.down, torch.cat([sh.full(m + "dq"), sh.full(m + "dkv"),
+                                    sh.full(m + "g")], 0), m + "dq|dkv|g")
+            put(mx.qnorm_w, sh.full(m + "dq.norm"), m + "dq.norm")
+            put(mx.kvnorm_w, sh.full(m + "dkv.norm"), m + "dkv.norm")
+            put(mx.uq, sh.full(m + "uq"), m + "uq")
+            put(mx.uk, sh.full(m + "uk").view(a.heads, a.dim, a.kv_rank),
+                m + "uk")
+            put(mx.uv_t, sh.full(m + "uv").view(
+                a.heads, a.vdim, a.kv_rank).transpose(1, 2), m + "uv")
+            put(mx.sink, sh.full(m + "sink"), m + "sink")
+            put(mx.o, sh.full(m + "o"), m + "o")
+        if spec.mlp is None:
+            continue
+        norm(layer.norm2, p + "norm2")
+        f, ff = layer.mlp, p + "mlp."
+        if isinstance(spec.mlp, DenseFFSpec):
+            put(f.up, sh.full(ff + "up"), ff + "up")
+            put(f.down, sh.full(ff + "down"), ff + "down")
+            put(f.act, sh.full(ff + "act"), ff + "act")
+        elif isinstance(spec.mlp, MoEFFSpec):
+            put(f.router_w, sh.full(ff + "router"), ff + "router")
+            put(f.router_b, sh.full(ff + "router.b"), ff + "router.b")
+            E = spec.mlp.experts
+            put(f.up_t, torch.stack(
+                [sh.full(ff + f"e{e}.up").t() for e in range(E)]),
+                ff + "e*.up")
+            put(f.down_t, torch.stack(
+                [sh.full(ff + f"e{e}.down").t() for e in range(E)]),
+                ff + "e*.down")
+            if f.shared_up is not None:
+                put(f.shared_up, sh.full(ff + "shared.up"),
+                    ff + "shared.up")
+                put(f.shared_down, sh.full(ff + "shared.down"),
+                    ff + "shared.down")
+    norm(model.final_norm, "final.norm")
+    put(model.head, sh.full("head"), "head")
+    return n
+
+
 def _is_gguf(path: str) -> bool:
     p = Path(path)
     if p.is_file():
@@ -275,6 +354,8 @@ def load_weights(model, path: str) -> int:
         from .gguf import load_gguf_weights
 
         return load_gguf_weights(model, path)
+    if getattr(model.cfg, "architecture", "") == "Fedatar":
+        return load_fedatar_weights(model, path)
     if getattr(model.cfg, "is_moe", False):
         return load_mixtral_weights(model, path)
     return load_llama_weights(model, path)

@@ -22,6 +22,24 @@ except ImportError:  # pragma: no cover - absent only before first build
     HAS_KERNELS = False
 
 
+try:
+    from . import _hybrid  # recurrent / latent-attention mechanisms
+
+    HAS_HYBRID = True
+except ImportError:  # pragma: no cover - absent only before first build
+    _hybrid = None
+    HAS_HYBRID = False
+
+
+def _require_hybrid() -> None:
+    if not HAS_HYBRID:
+        raise RuntimeError(
+            "inference_gateway_amd.ops._hybrid is not built but a GPU "
+            "tensor was passed. Build it in-tree with: IGW_BUILD_EXT=hybrid "
+            "PYTORCH_ROCM_ARCH=gfx950 python setup.py build_ext --inplace"
+        )
+
+
 def _require_kernels() -> None:
     if not HAS_KERNELS:
         raise RuntimeError(
@@ -150,6 +168,7 @@ def sample(logits, temperature, top_k, top_p, uniforms):
 
 
 build_cos_sin_cache = torch_ref.build_cos_sin_cache
+rotary_inv_freq = torch_ref.rotary_inv_freq
 make_prefill_tiles = torch_ref.make_prefill_tiles
 
 
@@ -228,3 +247,158 @@ def fused_gemm_tn_supported(M: int, N_rows: int, K: int,
                             swiglu: bool) -> bool:
     N = N_rows // 2 if swiglu else N_rows
     return M % 128 == 0 and N % 64 == 0 and K % 32 == 0
+
+
+# ---------------------------------------------------------------------------
+# Hybrid-decoder mechanisms: fp32-residual LayerNorm, minGRU scan, windowed
+# latent attention with a softmax sink, xIELU / relu^2 activations.  The
+# kernels are typed for bf16 AND fp32 activations (true 32-bit serving);
+# norms, recurrent state, angles and softmax are fp32 in both.
+# ---------------------------------------------------------------------------
+def add_layernorm(residual, delta, weight, bias, eps: float, out_dtype):
+    """residual [T, D] fp32 += delta (in place; delta may be None);
+    returns LayerNorm(residual) * weight + bias in out_dtype."""
+    if residual.is_cuda:
+        _require_hybrid()
+        out = torch.empty(residual.shape, dtype=out_dtype,
+                          device=residual.device)
+        _hybrid.add_layernorm(out, residual, delta, weight, bias, eps)
+        return out
+    return torch_ref.add_layernorm_ref(residual, delta, weight, bias, eps,
+                                       out_dtype)
+
+
+# rows per chunk of the chunked minGRU scan, and the segment length from
+# which it replaces the one-thread-per-channel walk
+MINGRU_CHUNK = 64
+MINGRU_CHUNKED_FROM = 256
+
+
+def mingru_scan(zug, state, seq_cu, seq_start, seq_slots, seq_rows):
+    """minGRU recurrence + output gate over a ragged batch.  zug [T, 3W]
+    (z | x | g pre-activations), state [slots, W] fp32 (read when the
+    sequence's first row is not position 0, always written back).
+    seq_rows: python row counts per sequence (host side; picks the
+    sequential or the chunked-scan schedule and lays out its chunks)."""
+    if zug.is_cuda:
+        _require_hybrid()
+        W = zug.shape[1] // 3
+        out = torch.empty((zug.shape[0], W), dtype=zug.dtype,
+                          device=zug.device)
+        if max(seq_rows) < MINGRU_CHUNKED_FROM:
+            _hybrid.mingru_scan(out, zug, state, seq_cu, seq_start,
+                                seq_slots)
+            return out
+        r0, r1, ccu, row = [], [], [0], 0
+        for n in seq_rows:
+            for a in range(0, n, MINGRU_CHUNK):
+                r0.append(row + a)
+                r1.append(row + min(n, a + MINGRU_CHUNK))
+            row += n
+            ccu.append(len(r0))
+        tab = torch.tensor([r0, r1], dtype=torch.int32).to(zug.device)
+        ccu_t = torch.tensor(ccu, dtype=torch.int32).to(zug.device)
+        work = torch.empty((2, len(r0), W), dtype=torch.float32,
+                           device=zug.device)
+        _hybrid.mingru_scan_chunked(out, zug, state, seq_start, seq_slots,
+                                    tab[0], tab[1], ccu_t, work)
+        return out
+    return torch_ref.mingru_scan_ref(zug, state, seq_cu, seq_start,
+                                     seq_slots)
+
+
+def rope_pairs_(x, positions, inv_freq, offset: int):
+    """In-place interleaved-pair rotation of x[T, H, hd][..., offset :
+    offset + 2*len(inv_freq)] by positions * inv_freq (fp32 angles)."""
+    if x.is_cuda:
+        _require_hybrid()
+        _hybrid.rope_pairs(x, positions, inv_freq, offset)
+        return x
+    return torch_ref.rope_pairs_ref(x, positions, inv_freq, offset)
+
+
+def latent_down_post(down, positions, slot_mapping, cache, qnorm_w,
+                     kvnorm_w, inv_freq, eps: float, q_rank: int,
+                     kv_rank: int, rot_dim: int, heads: int):
+    """Post-processing of the fused down projection [T, q_rank + kv_rank
+    + rot_dim + heads]: returns (normed query latent [T, q_rank],
+    sigmoid head gates [T, heads] fp32) and appends (normed latent |
+    rotated shared key) to the paged cache at slot_mapping."""
+    if down.is_cuda:
+        _require_hybrid()
+        T = down.shape[0]
+        cq = torch.empty((T, q_rank), dtype=down.dtype, device=down.device)
+        gate = torch.empty((T, heads), dtype=torch.float32,
+                           device=down.device)
+        _hybrid.latent_down_post(cq, gate, down, positions, slot_mapping,
+                                  cache, qnorm_w, kvnorm_w, inv_freq, eps,
+                                  q_rank, kv_rank, rot_dim, heads)
+        return cq, gate
+    return torch_ref.latent_down_post_ref(
+        down, positions, slot_mapping, cache, qnorm_w, kvnorm_w, inv_freq,
+        eps, q_rank, kv_rank, rot_dim, heads)
+
+
+def latent_attention(q_abs, q_rot, cache, block_table, row_seq, positions,
+                     sink, scale: float, window: int,
+                     num_prefill_rows: int = 0, prefill_seq_lens=None):
+    """Absorbed latent attention (all heads share one cached latent per
+    token) with a sliding window and a per-head softmax sink.
+    q_abs [T, H, kv_rank], q_rot [T, H, rot_dim] (strided views ok),
+    cache [blocks, block, kv_rank + rot_dim].  Rows [0, num_prefill_rows)
+    are prompt portions (tiled MFMA kernel; prefill_seq_lens = python
+    row counts per sequence), the rest are single decoded tokens."""
+    if q_abs.is_cuda:
+        _require_hybrid()
+        T, H, R = q_abs.shape
+        out = torch.empty((T, H, R), dtype=q_abs.dtype, device=q_abs.device)
+        _hybrid.latent_attention(out, q_abs, q_rot, cache, block_table,
+                                  row_seq, positions, sink, scale, window)
+        return out
+    return torch_ref.latent_attention_ref(
+        q_abs, q_rot, cache, block_table, row_seq, positions, sink, scale,
+        window)
+
+
+def xielu(z, pq):
+    if z.is_cuda:
+        _require_hybrid()
+        out = torch.empty_like(z)
+        _hybrid.xielu(out, z, pq)
+        return out
+    return torch_ref.xielu_ref(z, pq)
+
+
+def relu2(z):
+    if z.is_cuda:
+        _require_hybrid()
+        out = torch.empty_like(z)
+        _hybrid.relu2(out, z)
+        return out
+    return torch_ref.relu2_ref(z)
+
+
+def gate_heads(v, gate):
+    """v [H, T, vd] (strided ok), gate [T, H] fp32 -> [T, H*vd]."""
+    if v.is_cuda:
+        _require_hybrid()
+        H, T, vd = v.shape
+        out = torch.empty((T, H * vd), dtype=v.dtype, device=v.device)
+        _hybrid.gate_heads(out, v, gate)
+        return out
+    return torch_ref.gate_heads_ref(v, gate)
+
+
+def moe_topk_route(logits, top_k: int):
+    """logits [T, E] fp32 -> (softmax-over-chosen weights [T, K] fp32,
+    expert ids [T, K] int32); any K <= E <= 64 on the GPU kernel."""
+    if logits.is_cuda:
+        _require_hybrid()
+        T, E = logits.shape
+        w = torch.empty((T, top_k), dtype=torch.float32,
+                        device=logits.device)
+        idx = torch.empty((T, top_k), dtype=torch.int32,
+                          device=logits.device)
+        _hybrid.moe_topk_route(w, idx, logits)
+        return w, idx
+    return torch_ref.moe_topk_route_ref(logits, top_k)

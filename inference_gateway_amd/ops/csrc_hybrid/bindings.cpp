@@ -1,0 +1,58 @@
+// Python bindings for the hybrid-decoder kernel library (gfx950): the
+// mechanisms behind recurrent / latent-attention layers.  Built as its own
+// extension so a process that serves such a model compiles and loads only
+// these kernels.
+#include <torch/extension.h>
+
+namespace igw {
+void add_layernorm(torch::Tensor out, torch::Tensor residual,
+                   c10::optional<torch::Tensor> delta, torch::Tensor weight,
+                   torch::Tensor bias, double eps);
+void latent_down_post(torch::Tensor cq, torch::Tensor gate, torch::Tensor down,
+                      torch::Tensor positions, torch::Tensor slot_mapping,
+                      torch::Tensor cache, torch::Tensor qnorm_w,
+                      torch::Tensor kvnorm_w, torch::Tensor inv_freq,
+                      double eps, int64_t q_rank, int64_t kv_rank,
+                      int64_t rot_dim, int64_t heads);
+void rope_pairs(torch::Tensor x, torch::Tensor positions,
+                torch::Tensor inv_freq, int64_t offset);
+void xielu(torch::Tensor out, torch::Tensor in, torch::Tensor pq);
+void relu2(torch::Tensor out, torch::Tensor in);
+void gate_heads(torch::Tensor out, torch::Tensor v, torch::Tensor gate);
+void moe_topk_route(torch::Tensor weights, torch::Tensor idx,
+                    torch::Tensor logits);
+void mingru_scan(torch::Tensor y, torch::Tensor zug, torch::Tensor state,
+                 torch::Tensor seq_cu, torch::Tensor seq_start,
+                 torch::Tensor seq_slots);
+void mingru_scan_chunked(torch::Tensor y, torch::Tensor zug,
+                         torch::Tensor state, torch::Tensor seq_start,
+                         torch::Tensor seq_slots, torch::Tensor chunk_r0,
+                         torch::Tensor chunk_r1, torch::Tensor seq_chunk_cu,
+                         torch::Tensor work);
+void latent_attention(torch::Tensor out, torch::Tensor q_abs,
+                      torch::Tensor q_rot, torch::Tensor cache,
+                      torch::Tensor block_table, torch::Tensor row_seq,
+                      torch::Tensor positions, torch::Tensor sink,
+                      double scale, int64_t window);
+}  // namespace igw
+
+PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
+  m.def("add_layernorm", &igw::add_layernorm,
+        "fp32 residual += delta; LayerNorm with weight and bias");
+  m.def("latent_down_post", &igw::latent_down_post,
+        "latent RMS norms + shared-key rotation + paged append + head gates");
+  m.def("rope_pairs", &igw::rope_pairs,
+        "in-place interleaved-pair rotary on a slice of every head");
+  m.def("xielu", &igw::xielu, "xIELU activation");
+  m.def("relu2", &igw::relu2, "squared ReLU activation");
+  m.def("gate_heads", &igw::gate_heads,
+        "[H,T,vd] values times [T,H] gates -> [T,H*vd]");
+  m.def("moe_topk_route", &igw::moe_topk_route,
+        "top-k experts and softmax over the chosen logits");
+  m.def("mingru_scan", &igw::mingru_scan,
+        "minGRU recurrence, one thread per (sequence, channel)");
+  m.def("mingru_scan_chunked", &igw::mingru_scan_chunked,
+        "minGRU recurrence as a three-pass chunked scan");
+  m.def("latent_attention", &igw::latent_attention,
+        "absorbed latent attention, sliding window + softmax sink, paged");
+}

@@ -302,3 +302,153 @@ def silu_mul_grouped_ref(gate_up, counts, capacity):
             seg = gate_up[e * capacity:e * capacity + c]
             out[e * capacity:e * capacity + c] = silu_mul_ref(seg)
     return out
+
+
+# ---------------------------------------------------------------------------
+# Hybrid-decoder mechanisms (layer norm on an fp32 residual, minGRU scan,
+# windowed latent attention with a softmax sink, xIELU / relu^2).  These are
+# the CPU implementations behind ops.*; the GPU path runs the HIP kernels.
+# Everything the recurrences, norms, angles and softmax touch is fp32.
+# ---------------------------------------------------------------------------
+def add_layernorm_ref(residual, delta, w, b, eps, out_dtype):
+    """residual (fp32, in place) += delta; returns LayerNorm(residual)
+    with weight/bias, variance = mean squared deviation."""
+    if delta is not None:
+        residual.add_(delta.float())
+    mean = residual.mean(-1, keepdim=True)
+    dev = residual - mean
+    var = (dev * dev).mean(-1, keepdim=True)
+    return (dev * torch.rsqrt(var + eps) * w + b).to(out_dtype)
+
+
+def mingru_scan_ref(zug, state, seq_cu, seq_start, seq_slots):
+    """zug [T, 3W] = (gate pre-activation | candidate pre-activation |
+    output-gate pre-activation).  Per sequence and channel:
+    S <- (1 - z) S + z * cand, y = S * silu(g).  state [slots, W] fp32
+    carries S between steps; a sequence that starts at position 0 starts
+    from zero whatever its slot held."""
+    T, W3 = zug.shape
+    W = W3 // 3
+    x = zug.float()
+    z = torch.sigmoid(x[:, :W])
+    u = x[:, W:2 * W]
+    cand = torch.where(u >= 0, u + 0.5, torch.sigmoid(u))
+    a, bb = 1.0 - z, z * cand
+    g = x[:, 2 * W:]
+    out = torch.empty((T, W), dtype=torch.float32, device=zug.device)
+    cu = seq_cu.tolist()
+    starts = seq_start.tolist()
+    slots = seq_slots.tolist()
+    for s, slot in enumerate(slots):
+        S = (state[slot].clone() if starts[s] > 0
+             else torch.zeros(W, dtype=torch.float32, device=zug.device))
+        for t in range(cu[s], cu[s + 1]):
+            S = a[t] * S + bb[t]
+            out[t] = S
+        state[slot] = S
+    return (out * (g * torch.sigmoid(g))).to(zug.dtype)
+
+
+def _rope_pairs(x, positions, inv_freq):
+    """Interleaved pairs (2i, 2i+1) of the last dim of x [T, ..., 2n]
+    turned by positions * inv_freq[i]; fp32 in, fp32 out."""
+    ang = positions.float().unsqueeze(-1) * inv_freq.float()   # [T, n]
+    while ang.dim() < x.dim():
+        ang = ang.unsqueeze(1)
+    c, s = torch.cos(ang), torch.sin(ang)
+    u, v = x[..., 0::2], x[..., 1::2]
+    return torch.stack((u * c - v * s, v * c + u * s), -1).flatten(-2)
+
+
+def rope_pairs_ref(x, positions, inv_freq, offset):
+    """In place on x[..., offset : offset + 2*len(inv_freq)]."""
+    n2 = 2 * inv_freq.numel()
+    part = x[..., offset:offset + n2]
+    part.copy_(_rope_pairs(part.float(), positions, inv_freq).to(x.dtype))
+    return x
+
+
+def latent_down_post_ref(down, positions, slot_mapping, cache, qnorm_w,
+                         kvnorm_w, inv_freq, eps, q_rank, kv_rank, rot_dim,
+                         heads):
+    """Everything between the fused down projection and the up
+    projections: RMS-norm the query latent, RMS-norm the key/value
+    latent and write it with the rotated shared key into the paged
+    cache, and squash the per-head output gate."""
+    x = down.float()
+    cq = x[:, :q_rank]
+    cq = cq * torch.rsqrt((cq * cq).mean(-1, keepdim=True) + eps) * qnorm_w
+    c = x[:, q_rank:q_rank + kv_rank]
+    c = c * torch.rsqrt((c * c).mean(-1, keepdim=True) + eps) * kvnorm_w
+    kr = x[:, q_rank + kv_rank:q_rank + kv_rank + rot_dim].clone()
+    n2 = 2 * inv_freq.numel()
+    kr[:, :n2] = _rope_pairs(kr[:, :n2], positions, inv_freq)
+    flat = cache.view(-1, cache.shape[-1])
+    flat[slot_mapping.long()] = torch.cat([c, kr], -1).to(cache.dtype)
+    gate = torch.sigmoid(x[:, q_rank + kv_rank + rot_dim:
+                           q_rank + kv_rank + rot_dim + heads])
+    return cq.to(down.dtype), gate
+
+
+def latent_attention_ref(q_abs, q_rot, cache, block_table, row_seq,
+                         positions, sink, scale, window):
+    """Absorbed latent attention over the paged cache.  Row t of head h
+    scores key j as (q_abs[t,h] . c_j + q_rot[t,h] . kr_j) * scale for
+    pos-window < j <= pos; the softmax denominator also holds exp(sink_h).
+    Returns the probability-weighted sum of latents [T, H, kv_rank]."""
+    T, H, R = q_abs.shape
+    bs = cache.shape[1]
+    out = torch.zeros((T, H, R), dtype=torch.float32, device=q_abs.device)
+    pos = positions.tolist()
+    seqs = row_seq.tolist()
+    flat = cache.view(-1, cache.shape[-1])
+    qa, qr = q_abs.float(), q_rot.float()
+    for t in range(T):
+        p = pos[t]
+        lo = max(0, p - window + 1) if window > 0 else 0
+        j = torch.arange(lo, p + 1, device=q_abs.device)
+        bt = block_table[seqs[t]].long()
+        rows = flat[bt[j // bs] * bs + j % bs].float()        # [n, R+rd]
+        sc = (qa[t] @ rows[:, :R].t() + qr[t] @ rows[:, R:].t()) * scale
+        m = torch.maximum(sc.max(-1).values, sink)            # [H]
+        e = torch.exp(sc - m[:, None])
+        den = e.sum(-1) + torch.exp(sink - m)
+        out[t] = (e @ rows[:, :R]) / den[:, None]
+    return out.to(q_abs.dtype)
+
+
+def xielu_ref(z, pq):
+    """xIELU: softplus(p) z^2 + z/2 for z > 0, else
+    (1/2 + softplus(q)) (e^z - 1 - z) + z/2."""
+    x = z.float()
+    ap = torch.nn.functional.softplus(pq[0].float())
+    an = 0.5 + torch.nn.functional.softplus(pq[1].float())
+    neg = torch.clamp(x, max=0.0)
+    y = torch.where(x > 0, ap * x * x + 0.5 * x,
+                    an * (torch.expm1(neg) - neg) + 0.5 * x)
+    return y.to(z.dtype)
+
+
+def relu2_ref(z):
+    r = torch.relu(z.float())
+    return (r * r).to(z.dtype)
+
+
+def gate_heads_ref(v, gate):
+    """v [H, T, vd] per-head values, gate [T, H] fp32 -> [T, H*vd]."""
+    H, T, vd = v.shape
+    return (v.float().transpose(0, 1) * gate[:, :, None]).reshape(
+        T, H * vd).to(v.dtype)
+
+
+def moe_topk_route_ref(logits, top_k):
+    """Top-k experts by logit and the softmax over just those k."""
+    w, idx = torch.topk(logits, top_k, dim=-1)
+    return torch.softmax(w, dim=-1), idx.to(torch.int32)
+
+
+def rotary_inv_freq(base: float, dims: int, device="cpu"):
+    """f_i = base**(-2i/dims), i < dims/2, evaluated in float64 and
+    rounded once to fp32 (the angle position * f_i is an fp32 product)."""
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    return (float(base) ** (-2.0 * i / dims)).to(torch.float32).to(device)

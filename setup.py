@@ -21,22 +21,41 @@ CSRC = ROOT / "inference_gateway_amd" / "ops" / "csrc"
 sources = [str(CSRC / "bindings.cpp")] + sorted(
     str(p) for p in CSRC.glob("*.hip")
 )
+HYB = ROOT / "inference_gateway_amd" / "ops" / "csrc_hybrid"
+hybrid_sources = [str(HYB / "bindings.cpp")] + sorted(
+    str(p) for p in HYB.glob("*.hip")
+)
+
+# packed-fp32 instruction selection is switched off for all device code
+HIPCC_FLAGS = [
+    "-O3",
+    "-std=c++17",
+    "--offload-arch=gfx950",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+]
+
+
+def _ext(name, srcs):
+    return cpp_extension.CUDAExtension(
+        name=name,
+        sources=srcs,
+        extra_compile_args={"cxx": ["-O3", "-std=c++17"],
+                            "nvcc": list(HIPCC_FLAGS)},
+    )
+
+
+# IGW_BUILD_EXT=hybrid|kernels builds just one extension (a process that
+# serves one model family compiles only what it loads); default: both
+_which = os.environ.get("IGW_BUILD_EXT", "all")
+ext_modules = []
+if _which in ("all", "kernels"):
+    ext_modules.append(_ext("inference_gateway_amd.ops._kernels", sources))
+if _which in ("all", "hybrid"):
+    ext_modules.append(_ext("inference_gateway_amd.ops._hybrid",
+                            hybrid_sources))
 
 setup(
     name="inference_gateway_amd_kernels",
-    ext_modules=[
-        cpp_extension.CUDAExtension(
-            name="inference_gateway_amd.ops._kernels",
-            sources=sources,
-            extra_compile_args={
-                "cxx": ["-O3", "-std=c++17"],
-                "nvcc": [
-                    "-O3",
-                    "-std=c++17",
-                    "--offload-arch=gfx950",
-                ],
-            },
-        )
-    ],
+    ext_modules=ext_modules,
     cmdclass={"build_ext": cpp_extension.BuildExtension},
 )
