@@ -270,3 +270,18 @@ def save_checkpoint(path, cfg, W):
     save_file({k: v.contiguous() for k, v in W.items()},
               str(path / "model.safetensors"))
     return str(path)
+
+
+def absorbed_row(qa, qr, c, kr, pos, window, sink, scale):
+    """One query row of one head against cached rows c [n, R], kr [n, rd]
+    (row j = position j): the probability-weighted sum of latents, with
+    the sink in the denominator.  Plain loops, float64."""
+    lo = 0 if not window else max(0, pos - window + 1)
+    sc = [float((qa @ c[j] + qr @ kr[j]) * scale) for j in range(lo, pos + 1)]
+    mx = max(max(sc), float(sink))
+    e = [math.exp(s - mx) for s in sc]
+    den = sum(e) + math.exp(float(sink) - mx)
+    out = torch.zeros(c.shape[1], dtype=F64)
+    for n, j in enumerate(range(lo, pos + 1)):
+        out += e[n] / den * c[j]
+    return out
