@@ -339,6 +339,11 @@ def latent_down_post(down, positions, slot_mapping, cache, qnorm_w,
         eps, q_rank, kv_rank, rot_dim, heads)
 
 
+# bf16 batches run the MFMA tile kernel; off = the one-wave-per-row kernel
+# (any dtype, any sizes) for everything
+LATENT_ATTENTION_MFMA = True
+
+
 def latent_attention(q_abs, q_rot, cache, block_table, row_seq, positions,
                      sink, scale: float, window: int,
                      num_prefill_rows: int = 0, prefill_seq_lens=None):
@@ -352,8 +357,25 @@ def latent_attention(q_abs, q_rot, cache, block_table, row_seq, positions,
         _require_hybrid()
         T, H, R = q_abs.shape
         out = torch.empty((T, H, R), dtype=q_abs.dtype, device=q_abs.device)
+        if q_abs.dtype == torch.bfloat16 and LATENT_ATTENTION_MFMA:
+            tq = _hybrid.latent_attention_tile_rows(H)
+            row0, nrows, row = [], [], 0
+            for n in (prefill_seq_lens or []) if num_prefill_rows else []:
+                for a in range(0, n, tq):
+                    row0.append(row + a)
+                    nrows.append(min(tq, n - a))
+                row += n
+            assert row == num_prefill_rows
+            row0.extend(range(num_prefill_rows, T))
+            nrows.extend([1] * (T - num_prefill_rows))
+            tiles = torch.tensor([row0, nrows], dtype=torch.int32).to(
+                q_abs.device)
+            if _hybrid.latent_attention_mfma(
+                    out, q_abs, q_rot, cache, block_table, row_seq,
+                    positions, tiles[0], tiles[1], sink, scale, window):
+                return out
         _hybrid.latent_attention(out, q_abs, q_rot, cache, block_table,
-                                  row_seq, positions, sink, scale, window)
+                                 row_seq, positions, sink, scale, window)
         return out
     return torch_ref.latent_attention_ref(
         q_abs, q_rot, cache, block_table, row_seq, positions, sink, scale,

@@ -34,6 +34,13 @@ void latent_attention(torch::Tensor out, torch::Tensor q_abs,
                       torch::Tensor block_table, torch::Tensor row_seq,
                       torch::Tensor positions, torch::Tensor sink,
                       double scale, int64_t window);
+bool latent_attention_mfma(torch::Tensor out, torch::Tensor q_abs,
+                           torch::Tensor q_rot, torch::Tensor cache,
+                           torch::Tensor block_table, torch::Tensor row_seq,
+                           torch::Tensor positions, torch::Tensor tile_row0,
+                           torch::Tensor tile_nrows, torch::Tensor sink,
+                           double scale, int64_t window);
+int64_t latent_attention_tile_rows(int64_t H);
 }  // namespace igw
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -55,4 +62,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "minGRU recurrence as a three-pass chunked scan");
   m.def("latent_attention", &igw::latent_attention,
         "absorbed latent attention, sliding window + softmax sink, paged");
+  m.def("latent_attention_mfma", &igw::latent_attention_mfma,
+        "absorbed latent attention on MFMA tiles (bf16); false = sizes do "
+        "not fit, use latent_attention");
+  m.def("latent_attention_tile_rows", &igw::latent_attention_tile_rows,
+        "token rows per MFMA tile for a head count");
 }

@@ -629,3 +629,88 @@ def test_trace_runner_command(tmp_path):
         close(torch.tensor(a).view(2, V), ref[[0, len(t) - 2]], 2e-5)
         close(torch.tensor(b).view(1, V), ref[[len(t) - 1]], 2e-5)
     assert not (tmp_path / "out" / "10.f32").exists()
+
+
+# ---------------------------------------------------------------------------
+# GPU only: the bf16 matrix-core attention kernel against the plain
+# float64 rows, over its register-tile instantiations, both staging
+# paths, partial tiles, several head groups and ragged batches
+# ---------------------------------------------------------------------------
+@pytest.mark.gpu
+@pytest.mark.parametrize("R,RD,H,window", [
+    (20, 6, 3, 9),        # scalar staging, odd head count
+    (64, 16, 4, 0),       # vector staging, smallest tile set
+    (64, 16, 4, 37),
+    (136, 24, 100, 50),   # two head groups, middle tile set
+    (512, 64, 16, 70),    # largest tile set (LDS above 64 KiB)
+])
+def test_latent_attention_mfma(R, RD, H, window):
+    g = torch.Generator().manual_seed(31)
+    bs = 16
+    lens = [75, 130]                       # cached tokens per sequence
+    caches, tables = [], []
+    c_all, kr_all = [], []
+    nb_total = 1
+    for n in lens:
+        c = (torch.randn(n, R, generator=g) * 0.5).bfloat16().float()
+        kr = (torch.randn(n, RD, generator=g) * 0.5).bfloat16().float()
+        c_all.append(c)
+        kr_all.append(kr)
+    # interleave the two sequences' pages in one pool
+    nblk = [(n + bs - 1) // bs for n in lens]
+    perm = (torch.randperm(sum(nblk) + 2, generator=g) + 1).tolist()
+    cache = torch.randn(sum(nblk) + 4, bs, R + RD, generator=g)
+    flat = cache.view(-1, R + RD)
+    maxb = max(nblk)
+    bt = torch.zeros(2, maxb, dtype=torch.int32)
+    at = 0
+    for s, n in enumerate(lens):
+        pages = perm[at:at + nblk[s]]
+        at += nblk[s]
+        bt[s, :nblk[s]] = torch.tensor(pages, dtype=torch.int32)
+        for j in range(n):
+            flat[pages[j // bs] * bs + j % bs] = torch.cat(
+                [c_all[s][j], kr_all[s][j]])
+    # rows: a 23-row portion of seq 0 ending at its last token, a
+    # 41-row portion of seq 1 from position 60, then decoded rows
+    segs = [(0, 75 - 23, 23), (1, 60, 41)]
+    dec = [(1, 129), (0, 74)]
+    row_seq, pos = [], []
+    for s, p0, n in segs:
+        row_seq += [s] * n
+        pos += list(range(p0, p0 + n))
+    for s, p in dec:
+        row_seq.append(s)
+        pos.append(p)
+    T = len(pos)
+    qa = (torch.randn(T, H, R, generator=g) * 0.3).bfloat16()
+    qr = (torch.randn(T, H, RD, generator=g) * 0.3).bfloat16()
+    sink = torch.randn(H, generator=g)
+    scale = 0.7 / math.sqrt(R)
+    dev = "cuda"
+    out = ops.latent_attention(
+        qa.to(dev), qr.to(dev), cache.bfloat16().to(dev), bt.to(dev),
+        torch.tensor(row_seq, dtype=torch.int32, device=dev),
+        torch.tensor(pos, dtype=torch.int32, device=dev), sink.to(dev),
+        scale, window, 64, [23, 41]).float().cpu()
+    check_rows = [0, 1, 22, 23, 40, 63, 64, 65]
+    heads = sorted({0, H // 2, H - 1})
+    for t in check_rows:
+        s = row_seq[t]
+        for h in heads:
+            ref = oracle.absorbed_row(
+                qa[t, h].double(), qr[t, h].double(), c_all[s].double(),
+                kr_all[s].double(), pos[t], window, sink[h], scale)
+            torch.testing.assert_close(out[t, h].double(), ref, atol=2e-2,
+                                       rtol=2e-2)
+    # and the whole output against the fp32 one-wave-per-row kernel
+    ops.LATENT_ATTENTION_MFMA = False
+    try:
+        slow = ops.latent_attention(
+            qa.to(dev), qr.to(dev), cache.bfloat16().to(dev), bt.to(dev),
+            torch.tensor(row_seq, dtype=torch.int32, device=dev),
+            torch.tensor(pos, dtype=torch.int32, device=dev), sink.to(dev),
+            scale, window).float().cpu()
+    finally:
+        ops.LATENT_ATTENTION_MFMA = True
+    torch.testing.assert_close(out, slow, atol=2e-2, rtol=2e-2)
