@@ -78,6 +78,14 @@ def parse_args():
     ap.add_argument("--port", type=int, default=18300)
     ap.add_argument("--client-worker", action="store_true",
                     help=argparse.SUPPRESS)
+    ap.add_argument("--arch-compare", action="store_true",
+                    help="hybrid-decoder comparison instead of the "
+                         "serving benchmark: Fedatar beside Mixtral at "
+                         "equal layer sizes (engine prefill/decode "
+                         "tokens/s and per-kernel roofline fractions); "
+                         "prints its own JSON object")
+    ap.add_argument("--arch-size", type=str, default="2k",
+                    help="layer shape for --arch-compare (2k | 4k)")
     ap.add_argument("--num-gpu-blocks", type=int, default=0,
                     help=argparse.SUPPRESS)  # CPU smoke tests
     return ap.parse_args()
@@ -499,6 +507,15 @@ def main() -> None:
     args = parse_args()
     if args.client_worker:
         asyncio.run(client_worker_main(args))
+        return
+    if args.arch_compare:
+        sys.path.insert(0, str(Path(__file__).resolve().parent / "tools"))
+        import bench_hybrid
+
+        batch = args.batch if args.batch != 1024 else 64
+        print(json.dumps(bench_hybrid.run(
+            args.arch_size, batch, min(args.prompt_len, 1024), args.steps,
+            args.warmup)))
         return
     if args.tp or args.engine_only:
         bench_engine(args)

@@ -617,22 +617,32 @@ class LLMEngine:
         row -> sequence map (ForwardBatch.seq_*)."""
         dev = self.device
         S = len(seqs)
-        cu = [0]
-        for r in rows:
-            cu.append(cu[-1] + r)
-        maxb = max(len(s.block_ids) for s in seqs)
-        bt = torch.zeros((S, maxb), dtype=torch.int32)
-        for i, s in enumerate(seqs):
-            bt[i, : len(s.block_ids)] = torch.tensor(s.block_ids,
-                                                     dtype=torch.int32)
-        fb.seq_cu = torch.tensor(cu, dtype=torch.int32, device=dev)
-        fb.seq_start = torch.tensor(starts, dtype=torch.int32, device=dev)
         fb.seq_slots = torch.tensor([s.slot for s in seqs],
                                     dtype=torch.int32, device=dev)
-        fb.seq_block_table = bt.to(dev)
-        fb.row_seq = torch.repeat_interleave(
-            torch.arange(S, dtype=torch.int32),
-            torch.tensor(rows, dtype=torch.int64)).to(dev)
+        fb.max_context = max(s.num_tokens for s in seqs)
+        if not fb.is_prefill:
+            # pure decode: one row per sequence — the batch's own
+            # tensors already are the sequence-level view
+            ar = torch.arange(S + 1, dtype=torch.int32, device=dev)
+            fb.seq_cu, fb.row_seq = ar, ar[:S]
+            fb.seq_start = fb.positions
+            fb.seq_block_table = fb.block_table
+        else:
+            cu = [0]
+            for r in rows:
+                cu.append(cu[-1] + r)
+            maxb = max(len(s.block_ids) for s in seqs)
+            bt = torch.zeros((S, maxb), dtype=torch.int32)
+            for i, s in enumerate(seqs):
+                bt[i, : len(s.block_ids)] = torch.tensor(
+                    s.block_ids, dtype=torch.int32)
+            fb.seq_cu = torch.tensor(cu, dtype=torch.int32, device=dev)
+            fb.seq_start = torch.tensor(starts, dtype=torch.int32,
+                                        device=dev)
+            fb.seq_block_table = bt.to(dev)
+            fb.row_seq = torch.repeat_interleave(
+                torch.arange(S, dtype=torch.int32),
+                torch.tensor(rows, dtype=torch.int64)).to(dev)
         fb.seq_rows = list(rows)
         fb.num_chunk_rows = num_chunk_rows
 

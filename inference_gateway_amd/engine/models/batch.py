@@ -47,6 +47,7 @@ class ForwardBatch:
     row_seq: Optional[torch.Tensor] = None         # [T] int32 seq of a row
     seq_rows: Optional[List[int]] = None           # python row counts
     num_chunk_rows: int = 0                        # rows in prompt portions
+    max_context: int = 0                           # longest sequence (host)
 
     @property
     def is_mixed(self) -> bool:

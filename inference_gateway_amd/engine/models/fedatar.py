@@ -151,7 +151,7 @@ class LatentAttention(nn.Module):
         o_lat = ops.latent_attention(
             q_abs.transpose(0, 1), q[:, :, dn:], cache, fb.seq_block_table,
             fb.row_seq, fb.positions, self.sink, sp.scale, sp.window,
-            fb.num_chunk_rows, fb.seq_lens)
+            fb.num_chunk_rows, fb.seq_lens, fb.max_context)
         v = torch.bmm(o_lat.transpose(0, 1), self.uv_t)           # [H,T,vd]
         return F.linear(ops.gate_heads(v, gate), self.o)
 

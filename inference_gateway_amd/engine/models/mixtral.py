@@ -301,36 +301,15 @@ class MixtralMoE(nn.Module):
     def _forward_sorted(self, x: torch.Tensor) -> torch.Tensor:
         """Per-expert contiguous GEMMs for prefill-size batches, where the
         padded path's E/K-fold FLOP overhead would be compute-bound."""
-        T, h = x.shape
+        from . import moe_common
+
         router_logits = self.router(x).float()            # [T, E]
         weights, topk_idx = torch.topk(router_logits, self.top_k, dim=-1)
-        weights = torch.softmax(weights, dim=-1).to(x.dtype)  # [T, K]
-        out = torch.zeros_like(x)
-        flat_expert = topk_idx.reshape(-1)                # [T*K]
-        flat_token = (
-            torch.arange(T, device=x.device)
-            .unsqueeze(1)
-            .expand(T, self.top_k)
-            .reshape(-1)
-        )
-        # sort tokens by expert so each expert runs one contiguous GEMM
-        order = torch.argsort(flat_expert, stable=True)
-        sorted_expert = flat_expert[order]
-        sorted_token = flat_token[order]
-        counts = torch.bincount(sorted_expert, minlength=self.num_experts)
-        counts_list = counts.tolist()
-        start = 0
-        for e, cnt in enumerate(counts_list):
-            if cnt == 0:
-                continue
-            toks = sorted_token[start:start + cnt]
-            xe = x.index_select(0, toks)
-            gu = F.linear(xe, self.gate_up[e])
-            ye = F.linear(ops.silu_mul(gu), self.down[e])
-            w = weights.reshape(-1)[order[start:start + cnt]].unsqueeze(1)
-            out.index_add_(0, toks, ye * w)
-            start += cnt
-        return out
+        weights = torch.softmax(weights, dim=-1)          # [T, K] fp32
+        # the sort-by-expert dispatch is shared with the other
+        # mixture-of-experts feed-forwards (models/moe_common.py)
+        return moe_common.experts_sorted(
+            x, weights, topk_idx, self.gate_up_t, self.down_t, ops.silu_mul)
 
 
 class MixtralLayer(nn.Module):

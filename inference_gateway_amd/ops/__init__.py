@@ -270,7 +270,7 @@ def add_layernorm(residual, delta, weight, bias, eps: float, out_dtype):
 
 # rows per chunk of the chunked minGRU scan, and the segment length from
 # which it replaces the one-thread-per-channel walk
-MINGRU_CHUNK = 64
+MINGRU_CHUNK = 16
 MINGRU_CHUNKED_FROM = 256
 
 
@@ -289,16 +289,8 @@ def mingru_scan(zug, state, seq_cu, seq_start, seq_slots, seq_rows):
             _hybrid.mingru_scan(out, zug, state, seq_cu, seq_start,
                                 seq_slots)
             return out
-        r0, r1, ccu, row = [], [], [0], 0
-        for n in seq_rows:
-            for a in range(0, n, MINGRU_CHUNK):
-                r0.append(row + a)
-                r1.append(row + min(n, a + MINGRU_CHUNK))
-            row += n
-            ccu.append(len(r0))
-        tab = torch.tensor([r0, r1], dtype=torch.int32).to(zug.device)
-        ccu_t = torch.tensor(ccu, dtype=torch.int32).to(zug.device)
-        work = torch.empty((2, len(r0), W), dtype=torch.float32,
+        tab, ccu_t = _scan_chunks(tuple(seq_rows), MINGRU_CHUNK, zug.device)
+        work = torch.empty((2, tab.shape[1], W), dtype=torch.float32,
                            device=zug.device)
         _hybrid.mingru_scan_chunked(out, zug, state, seq_start, seq_slots,
                                     tab[0], tab[1], ccu_t, work)
@@ -339,6 +331,42 @@ def latent_down_post(down, positions, slot_mapping, cache, qnorm_w,
         eps, q_rank, kv_rank, rot_dim, heads)
 
 
+import functools
+
+
+@functools.lru_cache(maxsize=256)
+def _attention_tiles(tq: int, num_prefill_rows: int, seq_lens: tuple,
+                     T: int, device):
+    """[2, ntiles] int32 (first row, row count) of the attention tiles:
+    prompt portions cut into runs of tq rows, decoded rows one each.
+    Cached: serving repeats the same batch shapes."""
+    row0, nrows, row = [], [], 0
+    for n in seq_lens:
+        for a in range(0, n, tq):
+            row0.append(row + a)
+            nrows.append(min(tq, n - a))
+        row += n
+    assert row == num_prefill_rows
+    row0.extend(range(num_prefill_rows, T))
+    nrows.extend([1] * (T - num_prefill_rows))
+    return torch.tensor([row0, nrows], dtype=torch.int32).to(device)
+
+
+@functools.lru_cache(maxsize=256)
+def _scan_chunks(seq_rows: tuple, chunk: int, device):
+    """Chunk table of the chunked minGRU scan: ([2, NC] row ranges,
+    [S+1] chunk offsets per sequence), cached per batch shape."""
+    r0, r1, ccu, row = [], [], [0], 0
+    for n in seq_rows:
+        for a in range(0, n, chunk):
+            r0.append(row + a)
+            r1.append(row + min(n, a + chunk))
+        row += n
+        ccu.append(len(r0))
+    return (torch.tensor([r0, r1], dtype=torch.int32).to(device),
+            torch.tensor(ccu, dtype=torch.int32).to(device))
+
+
 # bf16 batches run the MFMA tile kernel; off = the one-wave-per-row kernel
 # (any dtype, any sizes) for everything
 LATENT_ATTENTION_MFMA = True
@@ -346,33 +374,31 @@ LATENT_ATTENTION_MFMA = True
 
 def latent_attention(q_abs, q_rot, cache, block_table, row_seq, positions,
                      sink, scale: float, window: int,
-                     num_prefill_rows: int = 0, prefill_seq_lens=None):
+                     num_prefill_rows: int = 0, prefill_seq_lens=None,
+                     max_context: int = 0):
     """Absorbed latent attention (all heads share one cached latent per
     token) with a sliding window and a per-head softmax sink.
     q_abs [T, H, kv_rank], q_rot [T, H, rot_dim] (strided views ok),
     cache [blocks, block, kv_rank + rot_dim].  Rows [0, num_prefill_rows)
-    are prompt portions (tiled MFMA kernel; prefill_seq_lens = python
-    row counts per sequence), the rest are single decoded tokens."""
+    are prompt portions (prefill_seq_lens = python row counts per
+    sequence), the rest are single decoded tokens; max_context is a host
+    hint (longest sequence in the batch) for splitting keys over
+    workgroups."""
     if q_abs.is_cuda:
         _require_hybrid()
         T, H, R = q_abs.shape
         out = torch.empty((T, H, R), dtype=q_abs.dtype, device=q_abs.device)
         if q_abs.dtype == torch.bfloat16 and LATENT_ATTENTION_MFMA:
-            tq = _hybrid.latent_attention_tile_rows(H)
-            row0, nrows, row = [], [], 0
-            for n in (prefill_seq_lens or []) if num_prefill_rows else []:
-                for a in range(0, n, tq):
-                    row0.append(row + a)
-                    nrows.append(min(tq, n - a))
-                row += n
-            assert row == num_prefill_rows
-            row0.extend(range(num_prefill_rows, T))
-            nrows.extend([1] * (T - num_prefill_rows))
-            tiles = torch.tensor([row0, nrows], dtype=torch.int32).to(
-                q_abs.device)
+            tiles = _attention_tiles(
+                _hybrid.latent_attention_tile_rows(H), num_prefill_rows,
+                tuple(prefill_seq_lens or ()) if num_prefill_rows else (),
+                T, q_abs.device)
+            ctx = max_context or 4096
+            max_keys = min(window, ctx) if window > 0 else ctx
             if _hybrid.latent_attention_mfma(
                     out, q_abs, q_rot, cache, block_table, row_seq,
-                    positions, tiles[0], tiles[1], sink, scale, window):
+                    positions, tiles[0], tiles[1], sink, scale, window,
+                    max_keys):
                 return out
         _hybrid.latent_attention(out, q_abs, q_rot, cache, block_table,
                                  row_seq, positions, sink, scale, window)

@@ -31,6 +31,19 @@ struct Act<uint16_t> {
 // gates are specified in 32-bit; the fast __expf is ~2 ulp worse)
 DEVINLINE float sigmoid_f32(float x) { return 1.0f / (1.0f + expf(-x)); }
 
+// fp32 logistic on the hardware exp/rcp units (a few ulp): used where the
+// activations around it are bf16 and the exact version is the bottleneck
+DEVINLINE float sigmoid_fast(float x) {
+  return __frcp_rn(1.0f + __expf(-x));
+}
+
+template <typename T>
+DEVINLINE float sigmoid_for(float x);
+template <>
+DEVINLINE float sigmoid_for<float>(float x) { return sigmoid_f32(x); }
+template <>
+DEVINLINE float sigmoid_for<uint16_t>(float x) { return sigmoid_fast(x); }
+
 #define IGW_DISPATCH_ACT(TENSOR, ...)                                   \
   do {                                                                  \
     if ((TENSOR).scalar_type() == torch::kBFloat16) {                   \

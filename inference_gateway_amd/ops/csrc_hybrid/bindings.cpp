@@ -39,7 +39,7 @@ bool latent_attention_mfma(torch::Tensor out, torch::Tensor q_abs,
                            torch::Tensor block_table, torch::Tensor row_seq,
                            torch::Tensor positions, torch::Tensor tile_row0,
                            torch::Tensor tile_nrows, torch::Tensor sink,
-                           double scale, int64_t window);
+                           double scale, int64_t window, int64_t max_keys);
 int64_t latent_attention_tile_rows(int64_t H);
 }  // namespace igw
 

@@ -28,16 +28,18 @@ typedef __attribute__((ext_vector_type(4))) float float4v;
 constexpr int LA_BN = 32;        // keys per tile
 constexpr int LA_PAD = 8;        // bf16 elements of row padding in LDS
 
-template <int KS, int NT>
+template <int KS, int NT, bool PIPE>
 __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
-    uint16_t* __restrict__ out, const uint16_t* __restrict__ q_abs,
+    uint16_t* __restrict__ out, float* __restrict__ part_o,
+    float* __restrict__ part_ml, int nsplit, int T, const uint16_t* __restrict__ q_abs,
     int64_t qa_s0, int64_t qa_s1, const uint16_t* __restrict__ q_rot,
     int64_t qr_s0, int64_t qr_s1, const uint16_t* __restrict__ cache,
     const int32_t* __restrict__ block_table, int max_blocks,
     const int32_t* __restrict__ row_seq, const int32_t* __restrict__ positions,
     const int32_t* __restrict__ tile_row0,
     const int32_t* __restrict__ tile_nrows, const float* __restrict__ sink,
-    float scale, int window, int H, int R, int RD, int block_size, int HB) {
+    float scale, int window, int H, int R, int RD, int block_size, int HB,
+    bool qvec) {
   extern __shared__ __attribute__((aligned(16))) uint16_t la_smem[];
   const int CW = R + RD;
   const int ks_n = (CW + 31) / 32;          // 32-wide steps actually used
@@ -55,8 +57,15 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
   const int h0 = blockIdx.y * HB;
   const int p0 = positions[row0];
   const int32_t* bt = block_table + (int64_t)row_seq[row0] * max_blocks;
-  const int hi = p0 + nrows - 1;
-  const int lo = window > 0 ? max(0, p0 - window + 1) : 0;
+  const int hi_all = p0 + nrows - 1;
+  const int lo_all = window > 0 ? max(0, p0 - window + 1) : 0;
+  // key splits (gridDim.z): each takes a contiguous run of whole key tiles;
+  // split 0 carries the sink
+  const int split = blockIdx.z;
+  const int ntile_all = (hi_all - lo_all) / LA_BN + 1;
+  const int per = (ntile_all + nsplit - 1) / nsplit;
+  const int lo = lo_all + split * per * LA_BN;
+  const int hi = min(hi_all, lo + per * LA_BN - 1);
 
   const int frag_m = lane & 15, frag_k8 = (lane >> 4) * 8;
   const int crow0 = (lane >> 4) * 4, ccol = lane & 15;
@@ -80,7 +89,13 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
 #pragma unroll
     for (int kk = 0; kk < KS; ++kk) {
       short8v f = {0, 0, 0, 0, 0, 0, 0, 0};
-      if (ok && kk < ks_n) {
+      if (qvec) {
+        // 8 entries never straddle q_abs | q_rot when R % 8 == 0: one
+        // 16-byte load per step, all steps in flight together
+        const int d = kk * 32 + frag_k8;
+        if (ok && d < CW)
+          f = *reinterpret_cast<const short8v*>(d < R ? qa + d : qr + (d - R));
+      } else if (ok && kk < ks_n) {
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
           const int d = kk * 32 + frag_k8 + e;
@@ -103,44 +118,73 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
     const int r = m / HB, hh = m % HB;
     const bool ok = r < nrows && h0 + hh < H;
     rpos[r4] = ok ? p0 + r : -1;           // -1: sees no key
-    m_run[r4] = ok ? sink[h0 + hh] : 0.0f;
-    l_run[r4] = 1.0f;
+    // later splits start empty: a finite "minus infinity" keeps the
+    // rescaling factors well defined
+    m_run[r4] = !ok ? 0.0f : split == 0 ? sink[h0 + hh] : -1e30f;
+    l_run[r4] = split == 0 ? 1.0f : 0.0f;
   }
   float4v acc_o[NT];
 #pragma unroll
   for (int nt = 0; nt < NT; ++nt) acc_o[nt] = {0.f, 0.f, 0.f, 0.f};
+  // pairs are numbered rows-major, so a wave is live iff its first pair is
+  const bool wave_live =
+      (wave * 16) / HB < nrows && h0 + (wave * 16) % HB < H;
 
+  // Staging.  256 % LA_BN == 0, so a thread stages the SAME key of every
+  // tile (key = tid % 32) and walks the row in 16-byte pieces 8 keys' worth
+  // of threads apart: one block-table lookup per tile per thread, and all of
+  // a tile's loads are issued together into registers.  The next tile's
+  // loads are issued BEFORE the current tile's matrix work, so memory
+  // latency hides behind the MFMAs (register double buffering).
   const bool vec = (CW % 8 == 0) && (R % 8 == 0);
+  constexpr int NCH = (KS + 1) / 2;      // 16-byte pieces per thread, max
+  const int skey = tid % LA_BN, spiece = tid / LA_BN;   // piece = 8*i + spiece
+  const int c8n = CW / 8;
+  ushort8 stage[NCH];
+  auto cached_row = [&](int j0) -> int64_t {
+    const int j = min(j0 + skey, hi);
+    return (int64_t)bt[j / block_size] * block_size + j % block_size;
+  };
+  auto issue_loads = [&](int j0) {
+    const uint16_t* row = cache + cached_row(j0) * CW;
+#pragma unroll
+    for (int i = 0; i < NCH; ++i) {
+      const int piece = i * (256 / LA_BN) + spiece;
+      if (piece < c8n)
+        stage[i] = *reinterpret_cast<const ushort8*>(row + piece * 8);
+    }
+  };
+  if (PIPE && vec && lo <= hi) issue_loads(lo);
+
   for (int j0 = lo; j0 <= hi; j0 += LA_BN) {
+    if (!PIPE && vec) issue_loads(j0);
     __syncthreads();   // previous tile consumed (and the zero fill landed)
     // ---- stage 32 cached rows: row-major for S, transposed for O ----
     if (vec) {
-      const int c8n = CW / 8;
-      for (int idx = tid; idx < LA_BN * c8n; idx += 256) {
-        const int key = idx / c8n, d8 = (idx % c8n) * 8;
-        const int j = min(j0 + key, hi);
-        const int64_t prow = (int64_t)bt[j / block_size] * block_size +
-                             j % block_size;
-        const ushort8 val =
-            *reinterpret_cast<const ushort8*>(cache + prow * CW + d8);
-        *reinterpret_cast<ushort8*>(k_s + key * krs + d8) = val;
-        if (d8 < R) {
 #pragma unroll
-          for (int e = 0; e < 8; ++e) ct_s[(d8 + e) * crs + key] = val.v[e];
+      for (int i = 0; i < NCH; ++i) {
+        const int d8 = (i * (256 / LA_BN) + spiece) * 8;
+        if (d8 < CW) {
+          *reinterpret_cast<ushort8*>(k_s + skey * krs + d8) = stage[i];
+          if (d8 < R) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e)
+              ct_s[(d8 + e) * crs + skey] = stage[i].v[e];
+          }
         }
       }
     } else {
-      for (int idx = tid; idx < LA_BN * CW; idx += 256) {
-        const int key = idx / CW, d = idx % CW;
-        const int j = min(j0 + key, hi);
-        const int64_t prow = (int64_t)bt[j / block_size] * block_size +
-                             j % block_size;
-        const uint16_t val = cache[prow * CW + d];
-        k_s[key * krs + d] = val;
-        if (d < R) ct_s[d * crs + key] = val;
+      const uint16_t* row = cache + cached_row(j0) * CW;
+      for (int d = spiece; d < CW; d += 256 / LA_BN) {
+        const uint16_t val = row[d];
+        k_s[skey * krs + d] = val;
+        if (d < R) ct_s[d * crs + skey] = val;
       }
     }
     __syncthreads();
+    if (PIPE && vec && j0 + LA_BN <= hi) issue_loads(j0 + LA_BN);
+
+    if (!wave_live) continue;   // no valid pair in this wave: stage only
 
     // ---- S = Q . K^T : two 16-key sub-tiles ----
     float4v acc_s[2];
@@ -205,19 +249,57 @@ __global__ __launch_bounds__(256) void latent_attention_mfma_kernel(
     }
   }
 
-  // ---- normalise and store the valid pairs ----
+  // ---- store the valid pairs: normalised, or as a partial to merge ----
 #pragma unroll
   for (int r4 = 0; r4 < 4; ++r4) {
     if (rpos[r4] < 0) continue;
     const int m = wave * 16 + crow0 + r4;
     const int r = m / HB, hh = m % HB;
-    const float inv = 1.0f / l_run[r4];
-    uint16_t* o = out + ((int64_t)(row0 + r) * H + h0 + hh) * R;
+    const int64_t pair = (int64_t)(row0 + r) * H + h0 + hh;
+    if (nsplit == 1) {
+      const float inv = 1.0f / l_run[r4];
+      uint16_t* o = out + pair * R;
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
-      const int d = nt * 16 + ccol;
-      if (nt < nt_n && d < R) o[d] = f32_to_bf16(acc_o[nt][r4] * inv);
+      for (int nt = 0; nt < NT; ++nt) {
+        const int d = nt * 16 + ccol;
+        if (nt < nt_n && d < R) o[d] = f32_to_bf16(acc_o[nt][r4] * inv);
+      }
+    } else {
+      const int64_t slot = (int64_t)split * T * H + pair;
+      float* o = part_o + slot * R;
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        const int d = nt * 16 + ccol;
+        if (nt < nt_n && d < R) o[d] = acc_o[nt][r4];
+      }
+      if (ccol == 0) {
+        part_ml[2 * slot] = m_run[r4];
+        part_ml[2 * slot + 1] = l_run[r4];
+      }
     }
+  }
+}
+
+// merge the key splits of one (row, head): out = sum_z acc_z e^(m_z - M) /
+// sum_z l_z e^(m_z - M)
+__global__ __launch_bounds__(64) void latent_attention_merge_kernel(
+    uint16_t* __restrict__ out, const float* __restrict__ part_o,
+    const float* __restrict__ part_ml, int nsplit, int64_t pairs, int R) {
+  const int64_t pair = blockIdx.x;
+  float M = -INFINITY;
+  for (int z = 0; z < nsplit; ++z)
+    M = fmaxf(M, part_ml[2 * (z * pairs + pair)]);
+  float den = 0.0f;
+  for (int z = 0; z < nsplit; ++z)
+    den += part_ml[2 * (z * pairs + pair) + 1] *
+           expf(part_ml[2 * (z * pairs + pair)] - M);
+  const float inv = 1.0f / den;
+  for (int d = threadIdx.x; d < R; d += 64) {
+    float acc = 0.0f;
+    for (int z = 0; z < nsplit; ++z)
+      acc += part_o[(z * pairs + pair) * R + d] *
+             expf(part_ml[2 * (z * pairs + pair)] - M);
+    out[pair * R + d] = f32_to_bf16(acc * inv);
   }
 }
 
@@ -236,7 +318,7 @@ bool latent_attention_mfma(torch::Tensor out, torch::Tensor q_abs,
                            torch::Tensor block_table, torch::Tensor row_seq,
                            torch::Tensor positions, torch::Tensor tile_row0,
                            torch::Tensor tile_nrows, torch::Tensor sink,
-                           double scale, int64_t window) {
+                           double scale, int64_t window, int64_t max_keys) {
   TORCH_CHECK(q_abs.is_cuda() && q_abs.dim() == 3 && q_abs.stride(2) == 1 &&
               q_abs.dtype() == torch::kBFloat16);
   TORCH_CHECK(q_rot.dim() == 3 && q_rot.stride(2) == 1 &&
@@ -273,16 +355,47 @@ bool latent_attention_mfma(torch::Tensor out, torch::Tensor q_abs,
                         dev);
   if ((int64_t)shmem > (int64_t)lds_max) return false;
   hipStream_t stream = at::cuda::getCurrentCUDAStream();
-  dim3 grid(ntiles, (H + HB - 1) / HB);
-#define LAUNCH_LA(KSV, NTV)                                                   \
+  const int hgroups = (H + HB - 1) / HB;
+  // Fewer workgroups than compute units (small decode batches): cut the
+  // keys into splits so the chip fills, at least 4 key tiles per split.
+  // Launches of up to a few workgroups per unit also prefetch the next key
+  // tile through registers; larger ones hide latency by themselves.
+  hipDeviceProp_t* prop = at::cuda::getCurrentDeviceProperties();
+  const int64_t cus = prop->multiProcessorCount;
+  const int64_t blocks = (int64_t)ntiles * hgroups;
+  int nsplit = 1;
+  if (blocks < cus) {
+    const int64_t key_tiles = std::max<int64_t>(1, max_keys / LA_BN);
+    nsplit = (int)std::min<int64_t>(
+        std::min<int64_t>(8, (cus + blocks - 1) / blocks),
+        std::max<int64_t>(1, key_tiles / 4));
+  }
+  const bool pipe = blocks * nsplit < 2048;
+  torch::Tensor part_o, part_ml;
+  if (nsplit > 1) {
+    auto f32 = q_abs.options().dtype(torch::kFloat32);
+    part_o = torch::empty({nsplit, (int64_t)T * H, R}, f32);
+    part_ml = torch::empty({nsplit, (int64_t)T * H, 2}, f32);
+  }
+  dim3 grid(ntiles, hgroups, nsplit);
+  // 16-byte query loads need aligned rows on both query tensors
+  const bool qvec =
+      R % 8 == 0 && RD % 8 == 0 && q_abs.stride(0) % 8 == 0 &&
+      q_abs.stride(1) % 8 == 0 && q_rot.stride(0) % 8 == 0 &&
+      q_rot.stride(1) % 8 == 0 &&
+      reinterpret_cast<uintptr_t>(q_abs.data_ptr()) % 16 == 0 &&
+      reinterpret_cast<uintptr_t>(q_rot.data_ptr()) % 16 == 0;
+#define LAUNCH_LA2(KSV, NTV, PIPEV)                                           \
   do {                                                                        \
-    auto kern = latent_attention_mfma_kernel<KSV, NTV>;                       \
+    auto kern = latent_attention_mfma_kernel<KSV, NTV, PIPEV>;                \
     if (shmem > 64 * 1024)                                                    \
       (void)hipFuncSetAttribute((const void*)kern,                            \
                                 hipFuncAttributeMaxDynamicSharedMemorySize,   \
                                 (int)shmem);                                  \
     hipLaunchKernelGGL(                                                       \
         kern, grid, dim3(256), shmem, stream, (uint16_t*)out.data_ptr(),      \
+        nsplit > 1 ? (float*)part_o.data_ptr() : nullptr,                     \
+        nsplit > 1 ? (float*)part_ml.data_ptr() : nullptr, nsplit, T,         \
         (const uint16_t*)q_abs.data_ptr(), (int64_t)q_abs.stride(0),          \
         (int64_t)q_abs.stride(1), (const uint16_t*)q_rot.data_ptr(),          \
         (int64_t)q_rot.stride(0), (int64_t)q_rot.stride(1),                   \
@@ -292,14 +405,28 @@ bool latent_attention_mfma(torch::Tensor out, torch::Tensor q_abs,
         (const int32_t*)positions.data_ptr(),                                 \
         (const int32_t*)tile_row0.data_ptr(),                                 \
         (const int32_t*)tile_nrows.data_ptr(), (const float*)sink.data_ptr(), \
-        (float)scale, (int)window, H, R, RD, (int)cache.size(1), HB);         \
+        (float)scale, (int)window, H, R, RD, (int)cache.size(1), HB, qvec);   \
+  } while (0)
+#define LAUNCH_LA(KSV, NTV)                                                   \
+  do {                                                                        \
+    if (pipe) LAUNCH_LA2(KSV, NTV, true);                                     \
+    else LAUNCH_LA2(KSV, NTV, false);                                         \
   } while (0)
   if (ks_n <= 4 && nt_n <= 4) LAUNCH_LA(4, 4);
   else if (ks_n <= 10 && nt_n <= 16) LAUNCH_LA(10, 16);
   else LAUNCH_LA(18, 32);
 #undef LAUNCH_LA
+#undef LAUNCH_LA2
   (void)hipGetLastError();   // a refused attribute must not poison the check
   HIP_CHECK_KERNEL();
+  if (nsplit > 1) {
+    hipLaunchKernelGGL(latent_attention_merge_kernel, dim3((int64_t)T * H),
+                       dim3(64), 0, stream, (uint16_t*)out.data_ptr(),
+                       (const float*)part_o.data_ptr(),
+                       (const float*)part_ml.data_ptr(), nsplit,
+                       (int64_t)T * H, R);
+    HIP_CHECK_KERNEL();
+  }
   return true;
 }
 

@@ -23,61 +23,124 @@ namespace igw {
 
 constexpr int GRU_BLOCK = 64;
 
-template <typename T>
-DEVINLINE void gru_coeffs(const T* row, int W, int c, float& a, float& b) {
-  const float z = sigmoid_f32(Act<T>::ld(row + c));
-  const float u = Act<T>::ld(row + W + c);
-  const float cand = u >= 0.0f ? u + 0.5f : sigmoid_f32(u);
-  a = 1.0f - z;
-  b = z * cand;
+// V consecutive channels per thread (V = 4 when the width and the row
+// stride allow 8/16-byte loads, else 1)
+template <typename T, int V>
+DEVINLINE void load_v(const T* p, float* o);
+template <>
+DEVINLINE void load_v<float, 1>(const float* p, float* o) { o[0] = *p; }
+template <>
+DEVINLINE void load_v<uint16_t, 1>(const uint16_t* p, float* o) {
+  o[0] = bf16_to_f32(*p);
+}
+template <>
+DEVINLINE void load_v<float, 4>(const float* p, float* o) {
+  const float4 v = *reinterpret_cast<const float4*>(p);
+  o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+}
+template <>
+DEVINLINE void load_v<uint16_t, 4>(const uint16_t* p, float* o) {
+  const ushort4x v = *reinterpret_cast<const ushort4x*>(p);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) o[i] = bf16_to_f32(v.v[i]);
+}
+template <typename T, int V>
+DEVINLINE void store_v(T* p, const float* o);
+template <>
+DEVINLINE void store_v<float, 1>(float* p, const float* o) { *p = o[0]; }
+template <>
+DEVINLINE void store_v<uint16_t, 1>(uint16_t* p, const float* o) {
+  *p = f32_to_bf16(o[0]);
+}
+template <>
+DEVINLINE void store_v<float, 4>(float* p, const float* o) {
+  *reinterpret_cast<float4*>(p) = make_float4(o[0], o[1], o[2], o[3]);
+}
+template <>
+DEVINLINE void store_v<uint16_t, 4>(uint16_t* p, const float* o) {
+  ushort4x v;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) v.v[i] = f32_to_bf16(o[i]);
+  *reinterpret_cast<ushort4x*>(p) = v;
 }
 
-template <typename T>
-DEVINLINE float gru_out(const T* row, int W, int c, float S) {
-  const float g = Act<T>::ld(row + 2 * W + c);
-  return S * (g * sigmoid_f32(g));
+template <typename T, int V>
+DEVINLINE void gru_coeffs(const T* row, int W, int c, float* a, float* b) {
+  float zp[V], u[V];
+  load_v<T, V>(row + c, zp);
+  load_v<T, V>(row + W + c, u);
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    const float z = sigmoid_for<T>(zp[i]);
+    const float cand = u[i] >= 0.0f ? u[i] + 0.5f : sigmoid_for<T>(u[i]);
+    a[i] = 1.0f - z;
+    b[i] = z * cand;
+  }
 }
 
-template <typename T>
+// one step of the recurrence for V channels; writes y = S * silu(g)
+template <typename T, int V>
+DEVINLINE void gru_step(const T* row, T* yrow, int W, int c, float* S) {
+  float a[V], b[V], g[V], y[V];
+  gru_coeffs<T, V>(row, W, c, a, b);
+  load_v<T, V>(row + 2 * W + c, g);
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    S[i] = a[i] * S[i] + b[i];
+    y[i] = S[i] * (g[i] * sigmoid_for<T>(g[i]));
+  }
+  store_v<T, V>(yrow + c, y);
+}
+
+template <typename T, int V>
 __global__ __launch_bounds__(GRU_BLOCK) void mingru_seq_kernel(
     T* __restrict__ y, const T* __restrict__ zug, int64_t zs,
     float* __restrict__ state, const int32_t* __restrict__ cu,
     const int32_t* __restrict__ start, const int32_t* __restrict__ slots,
     int W) {
   const int s = blockIdx.y;
-  const int c = blockIdx.x * GRU_BLOCK + threadIdx.x;
+  const int c = (blockIdx.x * GRU_BLOCK + threadIdx.x) * V;
   if (c >= W) return;
   const int r0 = cu[s], r1 = cu[s + 1];
   float* st = state + (int64_t)slots[s] * W + c;
-  float S = start[s] > 0 ? *st : 0.0f;
-  for (int r = r0; r < r1; ++r) {
-    const T* row = zug + (int64_t)r * zs;
-    float a, b;
-    gru_coeffs<T>(row, W, c, a, b);
-    S = a * S + b;
-    Act<T>::st(y + (int64_t)r * W + c, gru_out<T>(row, W, c, S));
-  }
-  *st = S;
+  float S[V];
+#pragma unroll
+  for (int i = 0; i < V; ++i) S[i] = start[s] > 0 ? st[i] : 0.0f;
+#pragma unroll 4
+  for (int r = r0; r < r1; ++r)
+    gru_step<T, V>(zug + (int64_t)r * zs, y + (int64_t)r * W, W, c, S);
+#pragma unroll
+  for (int i = 0; i < V; ++i) st[i] = S[i];
 }
 
 // pass 1: per chunk, P = prod a and Q = end state from a zero start
-template <typename T>
+template <typename T, int V>
 __global__ __launch_bounds__(GRU_BLOCK) void mingru_chunk_reduce_kernel(
     float* __restrict__ P, float* __restrict__ Q, const T* __restrict__ zug,
     int64_t zs, const int32_t* __restrict__ chunk_r0,
     const int32_t* __restrict__ chunk_r1, int W) {
   const int k = blockIdx.y;
-  const int c = blockIdx.x * GRU_BLOCK + threadIdx.x;
+  const int c = (blockIdx.x * GRU_BLOCK + threadIdx.x) * V;
   if (c >= W) return;
-  float p = 1.0f, q = 0.0f;
-  for (int r = chunk_r0[k]; r < chunk_r1[k]; ++r) {
-    float a, b;
-    gru_coeffs<T>(zug + (int64_t)r * zs, W, c, a, b);
-    p *= a;
-    q = a * q + b;
+  float p[V], q[V];
+#pragma unroll
+  for (int i = 0; i < V; ++i) { p[i] = 1.0f; q[i] = 0.0f; }
+  const int r1 = chunk_r1[k];
+#pragma unroll 4
+  for (int r = chunk_r0[k]; r < r1; ++r) {
+    float a[V], b[V];
+    gru_coeffs<T, V>(zug + (int64_t)r * zs, W, c, a, b);
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      p[i] *= a[i];
+      q[i] = a[i] * q[i] + b[i];
+    }
   }
-  P[(int64_t)k * W + c] = p;
-  Q[(int64_t)k * W + c] = q;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    P[(int64_t)k * W + c + i] = p[i];
+    Q[(int64_t)k * W + c + i] = q[i];
+  }
 }
 
 // pass 2: carry the state across each sequence's chunks; Q[k] becomes the
@@ -102,23 +165,22 @@ __global__ __launch_bounds__(GRU_BLOCK) void mingru_chunk_carry_kernel(
 }
 
 // pass 3: replay each chunk from its entering state and write y
-template <typename T>
+template <typename T, int V>
 __global__ __launch_bounds__(GRU_BLOCK) void mingru_chunk_apply_kernel(
     T* __restrict__ y, const float* __restrict__ Sin,
     const T* __restrict__ zug, int64_t zs,
     const int32_t* __restrict__ chunk_r0,
     const int32_t* __restrict__ chunk_r1, int W) {
   const int k = blockIdx.y;
-  const int c = blockIdx.x * GRU_BLOCK + threadIdx.x;
+  const int c = (blockIdx.x * GRU_BLOCK + threadIdx.x) * V;
   if (c >= W) return;
-  float S = Sin[(int64_t)k * W + c];
-  for (int r = chunk_r0[k]; r < chunk_r1[k]; ++r) {
-    const T* row = zug + (int64_t)r * zs;
-    float a, b;
-    gru_coeffs<T>(row, W, c, a, b);
-    S = a * S + b;
-    Act<T>::st(y + (int64_t)r * W + c, gru_out<T>(row, W, c, S));
-  }
+  float S[V];
+#pragma unroll
+  for (int i = 0; i < V; ++i) S[i] = Sin[(int64_t)k * W + c + i];
+  const int r1 = chunk_r1[k];
+#pragma unroll 4
+  for (int r = chunk_r0[k]; r < r1; ++r)
+    gru_step<T, V>(zug + (int64_t)r * zs, y + (int64_t)r * W, W, c, S);
 }
 
 static void check_scan_args(torch::Tensor y, torch::Tensor zug,
@@ -144,16 +206,21 @@ void mingru_scan(torch::Tensor y, torch::Tensor zug, torch::Tensor state,
   const int W = zug.size(1) / 3, S = seq_slots.numel();
   if (S == 0 || zug.size(0) == 0) return;
   hipStream_t stream = at::cuda::getCurrentCUDAStream();
-  dim3 grid((W + GRU_BLOCK - 1) / GRU_BLOCK, S);
+  const bool v4 = W % 4 == 0 && zug.stride(0) % 4 == 0;
+#define LAUNCH_SEQ(V)                                                        \
+  hipLaunchKernelGGL((mingru_seq_kernel<act_t, V>),                          \
+                     dim3((W / V + GRU_BLOCK - 1) / GRU_BLOCK, S),           \
+                     dim3(GRU_BLOCK), 0, stream, (act_t*)y.data_ptr(),       \
+                     (const act_t*)zug.data_ptr(), (int64_t)zug.stride(0),   \
+                     (float*)state.data_ptr(),                               \
+                     (const int32_t*)seq_cu.data_ptr(),                      \
+                     (const int32_t*)seq_start.data_ptr(),                   \
+                     (const int32_t*)seq_slots.data_ptr(), W)
   IGW_DISPATCH_ACT(zug, {
-    hipLaunchKernelGGL((mingru_seq_kernel<act_t>), grid, dim3(GRU_BLOCK), 0,
-                       stream, (act_t*)y.data_ptr(),
-                       (const act_t*)zug.data_ptr(), (int64_t)zug.stride(0),
-                       (float*)state.data_ptr(),
-                       (const int32_t*)seq_cu.data_ptr(),
-                       (const int32_t*)seq_start.data_ptr(),
-                       (const int32_t*)seq_slots.data_ptr(), W);
+    if (v4) LAUNCH_SEQ(4);
+    else LAUNCH_SEQ(1);
   });
+#undef LAUNCH_SEQ
   HIP_CHECK_KERNEL();
 }
 
@@ -175,24 +242,33 @@ void mingru_scan_chunked(torch::Tensor y, torch::Tensor zug,
   hipStream_t stream = at::cuda::getCurrentCUDAStream();
   float* P = (float*)work.data_ptr();
   float* Q = P + (int64_t)NC * W;
-  const int cb = (W + GRU_BLOCK - 1) / GRU_BLOCK;
+  const bool v4 = W % 4 == 0 && zug.stride(0) % 4 == 0;
+  const int cb1 = (W + GRU_BLOCK - 1) / GRU_BLOCK;
+#define LAUNCH_CHUNKED(V)                                                    \
+  do {                                                                       \
+    const int cb = (W / V + GRU_BLOCK - 1) / GRU_BLOCK;                      \
+    hipLaunchKernelGGL((mingru_chunk_reduce_kernel<act_t, V>), dim3(cb, NC), \
+                       dim3(GRU_BLOCK), 0, stream, P, Q,                     \
+                       (const act_t*)zug.data_ptr(), (int64_t)zug.stride(0), \
+                       (const int32_t*)chunk_r0.data_ptr(),                  \
+                       (const int32_t*)chunk_r1.data_ptr(), W);              \
+    hipLaunchKernelGGL(mingru_chunk_carry_kernel, dim3(cb1, S),              \
+                       dim3(GRU_BLOCK), 0, stream, P, Q,                     \
+                       (float*)state.data_ptr(),                             \
+                       (const int32_t*)seq_chunk_cu.data_ptr(),              \
+                       (const int32_t*)seq_start.data_ptr(),                 \
+                       (const int32_t*)seq_slots.data_ptr(), W);             \
+    hipLaunchKernelGGL((mingru_chunk_apply_kernel<act_t, V>), dim3(cb, NC),  \
+                       dim3(GRU_BLOCK), 0, stream, (act_t*)y.data_ptr(), Q,  \
+                       (const act_t*)zug.data_ptr(), (int64_t)zug.stride(0), \
+                       (const int32_t*)chunk_r0.data_ptr(),                  \
+                       (const int32_t*)chunk_r1.data_ptr(), W);              \
+  } while (0)
   IGW_DISPATCH_ACT(zug, {
-    hipLaunchKernelGGL((mingru_chunk_reduce_kernel<act_t>), dim3(cb, NC),
-                       dim3(GRU_BLOCK), 0, stream, P, Q,
-                       (const act_t*)zug.data_ptr(), (int64_t)zug.stride(0),
-                       (const int32_t*)chunk_r0.data_ptr(),
-                       (const int32_t*)chunk_r1.data_ptr(), W);
-    hipLaunchKernelGGL(mingru_chunk_carry_kernel, dim3(cb, S), dim3(GRU_BLOCK),
-                       0, stream, P, Q, (float*)state.data_ptr(),
-                       (const int32_t*)seq_chunk_cu.data_ptr(),
-                       (const int32_t*)seq_start.data_ptr(),
-                       (const int32_t*)seq_slots.data_ptr(), W);
-    hipLaunchKernelGGL((mingru_chunk_apply_kernel<act_t>), dim3(cb, NC),
-                       dim3(GRU_BLOCK), 0, stream, (act_t*)y.data_ptr(), Q,
-                       (const act_t*)zug.data_ptr(), (int64_t)zug.stride(0),
-                       (const int32_t*)chunk_r0.data_ptr(),
-                       (const int32_t*)chunk_r1.data_ptr(), W);
+    if (v4) LAUNCH_CHUNKED(4);
+    else LAUNCH_CHUNKED(1);
   });
+#undef LAUNCH_CHUNKED
   HIP_CHECK_KERNEL();
 }
 

@@ -229,9 +229,11 @@ class LocalProvider:
         weights = getattr(local_cfg, "weights_path", "") or None
         if local_cfg.model == "hf":
             # architecture straight from the checkpoint's config.json
-            from ..engine.weights import model_config_from_hf
+            # (HuggingFace Llama-family layouts, or the hybrid Fedatar
+            # design, which names itself in its config.json)
+            from ..engine.models.registry import model_config_from_dir
 
-            preset = model_config_from_hf(weights)
+            preset = model_config_from_dir(weights)
         elif local_cfg.model == "gguf":
             # architecture from GGUF metadata (llama.cpp checkpoints)
             from ..engine.gguf import model_config_from_gguf

@@ -99,11 +99,12 @@ def test_layernorm_residual(device, D):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("rows", [[5, 1, 9, 1], [300, 2], [1, 1, 1]])
-def test_mingru_scan(device, rows):
+@pytest.mark.parametrize("W", [37, 40])
+def test_mingru_scan(device, rows, W):
     """Ragged batch: fresh sequences (stale slot content must be
     ignored), continued ones (slot state is the start), and a segment
-    long enough for the chunked scan."""
-    W = 37
+    long enough for the chunked scan; widths with and without the
+    4-channel vector path."""
     g = torch.Generator().manual_seed(2)
     T, S = sum(rows), len(rows)
     zug = torch.randn(T, 3 * W, generator=g) * 2
@@ -714,3 +715,61 @@ def test_latent_attention_mfma(R, RD, H, window):
     finally:
         ops.LATENT_ATTENTION_MFMA = True
     torch.testing.assert_close(out, slow, atol=2e-2, rtol=2e-2)
+
+
+@pytest.mark.gpu
+def test_latent_attention_mfma_many_tiles():
+    """Thousands of single-row tiles: the launch shape that neither
+    splits keys nor prefetches through registers."""
+    g = torch.Generator().manual_seed(33)
+    R, RD, H, bs, n = 64, 16, 4, 16, 200
+    T = 2200
+    cache = (torch.randn(n // bs + 2, bs, R + RD, generator=g) * 0.5)
+    bt = (torch.randperm(n // bs + 1, generator=g) + 1).to(
+        torch.int32).view(1, -1)
+    pos = torch.randint(0, n, (T,), generator=g).to(torch.int32)
+    qa = (torch.randn(T, H, R, generator=g) * 0.3).bfloat16()
+    qr = (torch.randn(T, H, RD, generator=g) * 0.3).bfloat16()
+    sink = torch.randn(H, generator=g)
+    args = (qa.cuda(), qr.cuda(), cache.bfloat16().cuda(), bt.cuda(),
+            torch.zeros(T, dtype=torch.int32, device="cuda"), pos.cuda(),
+            sink.cuda(), 0.1, 70)
+    fast = ops.latent_attention(*args).float().cpu()
+    ops.LATENT_ATTENTION_MFMA = False
+    try:
+        slow = ops.latent_attention(*args).float().cpu()
+    finally:
+        ops.LATENT_ATTENTION_MFMA = True
+    torch.testing.assert_close(fast, slow, atol=2e-2, rtol=2e-2)
+
+
+def test_local_provider_serves_a_checkpoint_directory(tmp_path):
+    """The gateway's local provider with LOCAL_MODEL=hf picks the
+    architecture from the directory's config.json and generates through
+    the async engine."""
+    import asyncio
+
+    from inference_gateway_amd.config import LocalConfig
+    from inference_gateway_amd.providers.local import LocalProvider
+
+    cfg = oracle.make_config(vocab=300, pattern=("gd", "am"))
+    W = oracle.make_weights(cfg, seed=35)
+    path = oracle.save_checkpoint(tmp_path / "m", cfg, W)
+    lc = LocalConfig(enabled=True, model="hf", max_num_seqs=4,
+                     max_model_len=128)
+    lc.num_gpu_blocks = 64
+    lc.weights_path = path
+    provider = LocalProvider(lc, device="cpu")
+    try:
+        assert isinstance(provider.engine.engine.cfg.model, FedatarConfig)
+
+        async def go():
+            return await provider.chat_completions({
+                "model": "local/hf",
+                "messages": [{"role": "user", "content": "hi"}],
+                "max_tokens": 3, "temperature": 0})
+
+        body = asyncio.run(go())
+        assert body["usage"]["completion_tokens"] == 3
+    finally:
+        provider.engine.shutdown()
