@@ -52,7 +52,7 @@ def experts_sorted(x: torch.Tensor, weights: torch.Tensor,
                    down_t: torch.Tensor,
                    act: Callable[[torch.Tensor], torch.Tensor]
                    ) -> torch.Tensor:
-    """Same contract as experts_padded with topk_idx [T, K] instead of
+    """Same interface as experts_padded with topk_idx [T, K] instead of
     padded rows; per-expert contiguous GEMMs."""
     T, h = x.shape
     E = up_t.shape[0]

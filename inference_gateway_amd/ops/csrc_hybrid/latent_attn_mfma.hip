@@ -1,6 +1,6 @@
 // Absorbed latent attention on the matrix cores (gfx950, bf16).
 //
-// Same contract as latent_attention_rows (latent_attn.hip); this kernel is
+// Same interface as latent_attention_rows (latent_attn.hip); this kernel is
 // the serving path for bf16.  Because every head reads the SAME cached row
 // (latent | rotated key), heads are stacked into the M dimension of the MFMA
 // tiles: a workgroup owns 64 (token row, head) pairs — TQ consecutive rows

@@ -640,8 +640,8 @@ def test_trace_runner_command(tmp_path):
 @pytest.mark.gpu
 @pytest.mark.parametrize("R,RD,H,window", [
     (20, 6, 3, 9),        # scalar staging, odd head count
-    (64, 16, 4, 0),       # vector staging, smallest tile set
-    (64, 16, 4, 37),
+    (48, 16, 6, 0),       # vector staging, smallest tile set, key splits
+    (48, 16, 6, 37),
     (136, 24, 100, 50),   # two head groups, middle tile set
     (512, 64, 16, 70),    # largest tile set (LDS above 64 KiB)
 ])
@@ -722,7 +722,7 @@ def test_latent_attention_mfma_many_tiles():
     """Thousands of single-row tiles: the launch shape that neither
     splits keys nor prefetches through registers."""
     g = torch.Generator().manual_seed(33)
-    R, RD, H, bs, n = 64, 16, 4, 16, 200
+    R, RD, H, bs, n = 56, 8, 5, 16, 200
     T = 2200
     cache = (torch.randn(n // bs + 2, bs, R + RD, generator=g) * 0.5)
     bt = (torch.randperm(n // bs + 1, generator=g) + 1).to(
