@@ -215,10 +215,12 @@ class Relu2MoE(nn.Module):
         T = h.shape[0]
         E, K = self.spec.experts, self.spec.top
         logits = F.linear(h.float(), self.router_w, self.router_b)
-        weights, idx = ops.moe_topk_route(logits, K)
-        if T <= self.PADDED_MAX_ROWS:
-            C = (T + 63) // 64 * 64
-            dst = moe_common.padded_rows(idx, E, C)
+        padded = T <= self.PADDED_MAX_ROWS
+        C = (T + 63) // 64 * 64
+        weights, idx, dst = ops.moe_topk_route(logits, K, C if padded else 0)
+        if padded:
+            if dst is None:
+                dst = moe_common.padded_rows(idx, E, C)
             out = moe_common.experts_padded(h, weights, dst, self.up_t,
                                             self.down_t, C, ops.relu2)
         else:

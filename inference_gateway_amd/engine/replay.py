@@ -70,6 +70,8 @@ def run(engine, out_dir: str, lines, reply) -> None:
             if e["id"] not in ids:
                 ids[e["id"]] = engine.open_stream()
             sid = ids[e["id"]]
+            if not e["tokens"]:
+                continue             # admitted, nothing to run yet
             feeds.append((sid, e["tokens"]))
             want[sid] = e.get("want") or []
         n_want = sum(len(w) for w in want.values())

@@ -437,16 +437,25 @@ def gate_heads(v, gate):
     return torch_ref.gate_heads_ref(v, gate)
 
 
-def moe_topk_route(logits, top_k: int):
+def moe_topk_route(logits, top_k: int, capacity: int = 0):
     """logits [T, E] fp32 -> (softmax-over-chosen weights [T, K] fp32,
-    expert ids [T, K] int32); any K <= E <= 64 on the GPU kernel."""
-    if logits.is_cuda:
+    expert ids [T, K] int32, padded rows [T*K] int64 or None).  With
+    capacity > 0 (>= T) the padded-dispatch row of every assignment,
+    expert * capacity + rank, comes from the same launch.  Any K <= E <=
+    64 on the GPU kernel, wider routers take the library top-k."""
+    if logits.is_cuda and logits.shape[1] <= 64:
         _require_hybrid()
         T, E = logits.shape
         w = torch.empty((T, top_k), dtype=torch.float32,
                         device=logits.device)
         idx = torch.empty((T, top_k), dtype=torch.int32,
                           device=logits.device)
-        _hybrid.moe_topk_route(w, idx, logits)
-        return w, idx
-    return torch_ref.moe_topk_route_ref(logits, top_k)
+        dst = counts = None
+        if capacity > 0:
+            dst = torch.empty(T * top_k, dtype=torch.int64,
+                              device=logits.device)
+            counts = torch.zeros(E, dtype=torch.int32, device=logits.device)
+        _hybrid.moe_topk_route(w, idx, logits, dst, counts, capacity)
+        return w, idx, dst
+    w, idx = torch_ref.moe_topk_route_ref(logits, top_k)
+    return w, idx, None

@@ -20,7 +20,8 @@ void xielu(torch::Tensor out, torch::Tensor in, torch::Tensor pq);
 void relu2(torch::Tensor out, torch::Tensor in);
 void gate_heads(torch::Tensor out, torch::Tensor v, torch::Tensor gate);
 void moe_topk_route(torch::Tensor weights, torch::Tensor idx,
-                    torch::Tensor logits);
+                    torch::Tensor logits, c10::optional<torch::Tensor> dst,
+                    c10::optional<torch::Tensor> counts, int64_t capacity);
 void mingru_scan(torch::Tensor y, torch::Tensor zug, torch::Tensor state,
                  torch::Tensor seq_cu, torch::Tensor seq_start,
                  torch::Tensor seq_slots);

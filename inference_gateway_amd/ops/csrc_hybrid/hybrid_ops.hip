@@ -321,8 +321,10 @@ void gate_heads(torch::Tensor out, torch::Tensor v, torch::Tensor gate) {
 // lower expert id.
 __global__ void moe_topk_route_kernel(float* __restrict__ weights,
                                       int32_t* __restrict__ idx,
+                                      int64_t* __restrict__ dst,
+                                      int32_t* __restrict__ counts,
                                       const float* __restrict__ logits, int T,
-                                      int E, int K) {
+                                      int E, int K, int capacity) {
   const int t = blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= T) return;
   const float* row = logits + (int64_t)t * E;
@@ -352,10 +354,21 @@ __global__ void moe_topk_route_kernel(float* __restrict__ weights,
     z += e;
   }
   for (int k = 0; k < K; ++k) w[k] = w[k] / z;
+  // optional padded dispatch: row = expert * capacity + arrival rank (the
+  // order inside an expert's segment carries no meaning: the gather back
+  // uses the same rows)
+  if (dst != nullptr) {
+    for (int k = 0; k < K; ++k) {
+      const int e = id[k];
+      const int r = atomicAdd(counts + e, 1);
+      dst[(int64_t)t * K + k] = (int64_t)e * capacity + r;
+    }
+  }
 }
 
 void moe_topk_route(torch::Tensor weights, torch::Tensor idx,
-                    torch::Tensor logits) {
+                    torch::Tensor logits, c10::optional<torch::Tensor> dst,
+                    c10::optional<torch::Tensor> counts, int64_t capacity) {
   TORCH_CHECK(logits.is_cuda() && logits.dtype() == torch::kFloat32 &&
               logits.is_contiguous() && logits.dim() == 2);
   const int T = logits.size(0), E = logits.size(1), K = weights.size(1);
@@ -364,12 +377,21 @@ void moe_topk_route(torch::Tensor weights, torch::Tensor idx,
               weights.size(0) == T);
   TORCH_CHECK(idx.is_contiguous() && idx.dtype() == torch::kInt32 &&
               idx.size(0) == T && idx.size(1) == K);
+  if (dst.has_value()) {
+    TORCH_CHECK(counts.has_value() && capacity >= T);
+    TORCH_CHECK(dst->is_contiguous() && dst->dtype() == torch::kInt64 &&
+                dst->numel() == (int64_t)T * K);
+    TORCH_CHECK(counts->is_contiguous() && counts->dtype() == torch::kInt32 &&
+                counts->numel() == E);   // zeroed by the caller
+  }
   if (T == 0) return;
   hipStream_t stream = at::cuda::getCurrentCUDAStream();
   hipLaunchKernelGGL(moe_topk_route_kernel, dim3((T + 63) / 64), dim3(64), 0,
                      stream, (float*)weights.data_ptr(),
-                     (int32_t*)idx.data_ptr(), (const float*)logits.data_ptr(),
-                     T, E, K);
+                     (int32_t*)idx.data_ptr(),
+                     dst.has_value() ? (int64_t*)dst->data_ptr() : nullptr,
+                     dst.has_value() ? (int32_t*)counts->data_ptr() : nullptr,
+                     (const float*)logits.data_ptr(), T, E, K, (int)capacity);
   HIP_CHECK_KERNEL();
 }
 

@@ -251,13 +251,23 @@ def test_latent_attention_op(device, R, RD, H):
                                            rtol=3e-5)
 
 
-@pytest.mark.parametrize("device", DEVICES)
-def test_latent_attention_far_key_window_edges_and_sink(device):
+CRAFTED = [("cpu", "float32", "decode"), ("cpu", "float32", "prompt"),
+           pytest.param("cuda", "float32", "decode", marks=pytest.mark.gpu),
+           pytest.param("cuda", "bfloat16", "decode", marks=pytest.mark.gpu),
+           pytest.param("cuda", "bfloat16", "prompt", marks=pytest.mark.gpu)]
+
+
+@pytest.mark.parametrize("device,dtype,where", CRAFTED)
+def test_latent_attention_far_key_window_edges_and_sink(device, dtype,
+                                                        where):
     """Inputs shaped so that ONE key decides the result: a far key among
     hundreds (full attention), the oldest key a window still holds, and
     the first key it has dropped; and a dominant sink empties the
-    output."""
-    R, RD, bs, n = 16, 4, 16, 330
+    output.  The deciding query is either a lone decoded row or the last
+    row of a five-row prompt portion."""
+    R, RD, bs, n = 16, 8, 16, 330
+    dt = getattr(torch, dtype)
+    tol = 1e-3 if dt == torch.float32 else 5e-2
     g = torch.Generator().manual_seed(7)
     c = torch.randn(n, R, generator=g) * 0.1
     kr = torch.randn(n, RD, generator=g) * 0.1
@@ -265,50 +275,94 @@ def test_latent_attention_far_key_window_edges_and_sink(device):
     for j, axis in marks.items():      # distinctive keys on page borders
         c[j] = 0
         c[j, axis] = 6.0               # and just inside/outside a window
+    c, kr = c.to(dt).float(), kr.to(dt).float()
     cache, pages = _paged(c, kr, bs, 8)
     bt = torch.tensor([pages], dtype=torch.int32)
     pos = n - 1
+    nq = 1 if where == "decode" else 5
 
     def run(qvec, window, sink):
-        qa = torch.zeros(1, 1, R)
-        qa[0, 0] = qvec
+        qa = torch.randn(nq, 1, R, generator=g) * 0.1
+        qa[-1, 0] = qvec
         out = ops.latent_attention(
-            qa.to(device), torch.zeros(1, 1, RD, device=device),
-            cache.to(device), bt.to(device),
-            torch.zeros(1, dtype=torch.int32, device=device),
-            torch.tensor([pos], dtype=torch.int32, device=device),
-            torch.tensor([sink], device=device), 1.0, window)
-        return out[0, 0].cpu().double()
+            qa.to(dt).to(device),
+            torch.zeros(nq, 1, RD, dtype=dt, device=device),
+            cache.to(dt).to(device), bt.to(device),
+            torch.zeros(nq, dtype=torch.int32, device=device),
+            torch.arange(pos - nq + 1, pos + 1, dtype=torch.int32,
+                         device=device),
+            torch.tensor([sink], device=device), 1.0, window,
+            nq if where == "prompt" else 0,
+            [nq] if where == "prompt" else None)
+        return out[-1, 0].float().cpu().double()
 
     def unit(axis):
         v = torch.zeros(R)
         v[axis] = 6.0
         return v
 
+    def ref(axis, window, sink):
+        return oracle.absorbed_row(
+            unit(axis).double(), torch.zeros(RD).double(), c.double(),
+            kr.double(), pos, window, sink, 1.0)
+
     # far key, full attention: the output IS that latent
     torch.testing.assert_close(run(unit(0), 0, -30.0), c[17].double(),
-                               atol=1e-3, rtol=1e-3)
+                               atol=tol, rtol=tol)
     # window 40 ends at position 290 = n - 40: seen
     torch.testing.assert_close(run(unit(1), 40, -30.0), c[290].double(),
-                               atol=1e-3, rtol=1e-3)
+                               atol=tol, rtol=tol)
     # position 289 is one too old: the marked key must be invisible
     out = run(unit(2), 40, -30.0)
-    ref = oracle.absorbed_row(unit(2).double(), torch.zeros(RD).double(),
-                              c.double(), kr.double(), pos, 40, -30.0, 1.0)
-    torch.testing.assert_close(out, ref, atol=1e-4, rtol=1e-4)
+    torch.testing.assert_close(out, ref(2, 40, -30.0), atol=tol, rtol=tol)
     assert float(out[2]) < 1.0
     # keys on both sides of a page border
     torch.testing.assert_close(run(unit(3), 0, -30.0), c[255].double(),
-                               atol=1e-3, rtol=1e-3)
+                               atol=tol, rtol=tol)
     torch.testing.assert_close(run(unit(4), 0, -30.0), c[256].double(),
-                               atol=1e-3, rtol=1e-3)
+                               atol=tol, rtol=tol)
     # a huge sink takes all the mass and carries no value
     assert float(run(unit(0), 0, 80.0).abs().max()) < 1e-6
     # a moderate sink: exact share (the sink is not scaled, counts once)
-    out = run(unit(0), 0, 30.0)
-    ref = oracle.absorbed_row(unit(0).double(), torch.zeros(RD).double(),
-                              c.double(), kr.double(), pos, 0, 30.0, 1.0)
-    torch.testing.assert_close(out, ref, atol=1e-4, rtol=1e-4)
+    torch.testing.assert_close(run(unit(0), 0, 30.0), ref(0, 0, 30.0),
+                               atol=tol, rtol=tol)
+
+
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("T", [7, 300])
+def test_feed_forward_modules(device, T):
+    """Dense xIELU and routed relu^2 feed-forwards alone, through the
+    padded (few rows) and the sorted (many rows) expert dispatch."""
+    from inference_gateway_amd.engine.config import DenseFFSpec, MoEFFSpec
+    from inference_gateway_amd.engine.models.fedatar import (Relu2MoE,
+                                                             XieluMLP)
+
+    D = 24
+    cfg = oracle.make_config(width=D, pattern=("gd", "gm"), ff=20,
+                             experts=5, top=2, expert_ff=9, shared_ff=7)
+    W = {k: v.float() for k, v in oracle.make_weights(cfg, seed=37).items()}
+    h = torch.randn(T, D, generator=torch.Generator().manual_seed(38))
+    dev = _dev(device)
+    mlp = XieluMLP(D, DenseFFSpec(ff=20), "x", dev, torch.float32)
+    mlp.up.data.copy_(W["l0.mlp.up"])
+    mlp.down.data.copy_(W["l0.mlp.down"])
+    mlp.act.data.copy_(W["l0.mlp.act"])
+    W64 = {k: v.double() for k, v in W.items()}
+    close(mlp(h.to(dev), None), oracle.dense_ff(h.double(), W64, "l0.mlp."),
+          2e-5)
+    moe = Relu2MoE(D, MoEFFSpec(experts=5, top=2, expert_ff=9, shared_ff=7),
+                   "m", dev, torch.float32)
+    moe.router_w.data.copy_(W["l1.mlp.router"])
+    moe.router_b.data.copy_(W["l1.mlp.router.b"])
+    moe.up_t.data.copy_(torch.stack(
+        [W[f"l1.mlp.e{e}.up"].t() for e in range(5)]))
+    moe.down_t.data.copy_(torch.stack(
+        [W[f"l1.mlp.e{e}.down"].t() for e in range(5)]))
+    moe.shared_up.data.copy_(W["l1.mlp.shared.up"])
+    moe.shared_down.data.copy_(W["l1.mlp.shared.down"])
+    close(moe(h.to(dev), None),
+          oracle.moe_ff(h.double(), W64, "l1.mlp.", cfg["layers"][1]["mlp"]),
+          2e-5)
 
 
 @pytest.mark.parametrize("device", DEVICES)
@@ -325,8 +379,13 @@ def test_activations_and_route(device):
         torch.clamp(z.double(), min=0) ** 2, atol=1e-5, rtol=1e-5)
     for E, K in ((5, 3), (12, 12), (7, 1)):
         lg = torch.randn(19, E, generator=g)
-        w, idx = ops.moe_topk_route(lg.to(device), K)
+        w, idx, dst = ops.moe_topk_route(lg.to(device), K, 64)
         w, idx = w.cpu(), idx.cpu()
+        if dst is not None:
+            # padded rows: distinct, inside the chosen expert's segment
+            d = dst.cpu().view(19, K)
+            assert len(set(d.flatten().tolist())) == 19 * K
+            assert torch.equal(d // 64, idx.long())
         for t in range(19):
             order = sorted(range(E), key=lambda e: -float(lg[t, e]))[:K]
             assert idx[t].tolist() == order

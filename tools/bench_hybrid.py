@@ -244,7 +244,7 @@ def _kernels(sz):
 
     # ---- routing, 256 rows ----
     lg = torch.randn(256, sz["experts"], device=dev)
-    t = _time(lambda: ops.moe_topk_route(lg, sz["top"]))
+    t = _time(lambda: ops.moe_topk_route(lg, sz["top"], 256))
     out["moe_topk_route"] = _entry(t)
     t = _time(lambda: ops.moe_route(lg, sz["top"], 256))
     out["moe_route"] = _entry(t)
