@@ -31,8 +31,8 @@ typedef __attribute__((ext_vector_type(4))) float float4v;
 constexpr int LA_BN = 32;        // keys per tile
 constexpr int LA_PAD = 8;        // bf16 elements of row padding in LDS
 
-template <int KS, int NT, bool PIPE>
-__global__ __launch_bounds__(256, (KS <= 10 ? 2 : 1)) void latent_attention_mfma_kernel(
+template <int KS, int NT, bool PIPE, int NW>
+__global__ __launch_bounds__(NW * 64, ((NW == 4 && KS <= 10) ? 2 : 1)) void latent_attention_mfma_kernel(
     uint16_t* __restrict__ out, float* __restrict__ part_o,
     float* __restrict__ part_ml, int nsplit, int T, const uint16_t* __restrict__ q_abs,
     int64_t qa_s0, int64_t qa_s1, const uint16_t* __restrict__ q_rot,
@@ -51,7 +51,10 @@ __global__ __launch_bounds__(256, (KS <= 10 ? 2 : 1)) void latent_attention_mfma
   constexpr int crs = LA_BN + LA_PAD;       // CT / P row stride
   uint16_t* k_s = la_smem;                          // [32][krs]
   uint16_t* ct_s = k_s + LA_BN * krs;               // [nt_n*16][crs]
-  uint16_t* p_s = ct_s + nt_n * 16 * crs;           // [4][16][crs]
+  uint16_t* p_s = ct_s + nt_n * 16 * crs;           // [NW][16][crs]
+  constexpr int NTHR = NW * 64;   // NW = 4: 64 pairs per workgroup; NW = 1:
+                                  // one wave owns its 16 pairs and its key
+                                  // tiles alone (decode launches, few heads)
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   uint16_t* pw_s = p_s + wave * 16 * crs;
@@ -75,9 +78,9 @@ __global__ __launch_bounds__(256, (KS <= 10 ? 2 : 1)) void latent_attention_mfma
 
   // zero the LDS columns/rows that staging never writes (they meet zero
   // query padding, but stale bits could be NaN patterns)
-  for (int i = tid; i < LA_BN * krs; i += 256)
+  for (int i = tid; i < LA_BN * krs; i += NTHR)
     if (i % krs >= CW) k_s[i] = 0;
-  for (int i = tid; i < (nt_n * 16 - R) * crs; i += 256)
+  for (int i = tid; i < (nt_n * 16 - R) * crs; i += NTHR)
     ct_s[R * crs + i] = 0;
 
   // ---- Q fragments: A operand, row = pair (r, head), 8 entries of the
@@ -140,8 +143,9 @@ __global__ __launch_bounds__(256, (KS <= 10 ? 2 : 1)) void latent_attention_mfma
   // loads are issued BEFORE the current tile's matrix work, so memory
   // latency hides behind the MFMAs (register double buffering).
   const bool vec = (CW % 8 == 0) && (R % 8 == 0);
-  constexpr int NCH = (KS + 1) / 2;      // 16-byte pieces per thread, max
-  const int skey = tid % LA_BN, spiece = tid / LA_BN;   // piece = 8*i + spiece
+  constexpr int PSTEP = NTHR / LA_BN;    // pieces covered per pass
+  constexpr int NCH = (KS * 4 + PSTEP - 1) / PSTEP;   // pieces per thread
+  const int skey = tid % LA_BN, spiece = tid / LA_BN;
   const int c8n = CW / 8;
   ushort8 stage[NCH];
   auto cached_row = [&](int j0) -> int64_t {
@@ -152,7 +156,7 @@ __global__ __launch_bounds__(256, (KS <= 10 ? 2 : 1)) void latent_attention_mfma
     const uint16_t* row = cache + cached_row(j0) * CW;
 #pragma unroll
     for (int i = 0; i < NCH; ++i) {
-      const int piece = i * (256 / LA_BN) + spiece;
+      const int piece = i * PSTEP + spiece;
       if (piece < c8n)
         stage[i] = *reinterpret_cast<const ushort8*>(row + piece * 8);
     }
@@ -166,7 +170,7 @@ __global__ __launch_bounds__(256, (KS <= 10 ? 2 : 1)) void latent_attention_mfma
     if (vec) {
 #pragma unroll
       for (int i = 0; i < NCH; ++i) {
-        const int d8 = (i * (256 / LA_BN) + spiece) * 8;
+        const int d8 = (i * PSTEP + spiece) * 8;
         if (d8 < CW) {
           *reinterpret_cast<ushort8*>(k_s + skey * krs + d8) = stage[i];
           if (d8 < R) {
@@ -178,7 +182,7 @@ __global__ __launch_bounds__(256, (KS <= 10 ? 2 : 1)) void latent_attention_mfma
       }
     } else {
       const uint16_t* row = cache + cached_row(j0) * CW;
-      for (int d = spiece; d < CW; d += 256 / LA_BN) {
+      for (int d = spiece; d < CW; d += PSTEP) {
         const uint16_t val = row[d];
         k_s[skey * krs + d] = val;
         if (d < R) ct_s[d * crs + skey] = val;
@@ -307,7 +311,9 @@ __global__ __launch_bounds__(64) void latent_attention_merge_kernel(
 }
 
 // heads per workgroup and rows per tile for a head count
-static inline int la_heads_per_block(int H) { return H < 64 ? H : 64; }
+static inline int la_heads_per_block(int H, int nw = 4) {
+  return H < nw * 16 ? H : nw * 16;
+}
 
 int64_t latent_attention_tile_rows(int64_t H) {
   const int HB = la_heads_per_block((int)H);
@@ -346,11 +352,15 @@ bool latent_attention_mfma(torch::Tensor out, torch::Tensor q_abs,
   const int CW = R + RD;
   const int ks_n = (CW + 31) / 32, nt_n = (R + 15) / 16;
   if (ks_n > 18 || nt_n > 32) return false;
-  const int HB = la_heads_per_block(H);
+  // decode-only launches with few heads: single-wave workgroups (no idle
+  // waves, no cross-wave barriers, three per compute unit by LDS)
+  const int nw =
+      (ntiles == T && H <= 32 && ks_n <= 10 && nt_n <= 16) ? 1 : 4;
+  const int HB = la_heads_per_block(H, nw);
   const size_t shmem =
       sizeof(uint16_t) * ((size_t)LA_BN * (ks_n * 32 + LA_PAD) +
                           (size_t)nt_n * 16 * (LA_BN + LA_PAD) +
-                          (size_t)4 * 16 * (LA_BN + LA_PAD));
+                          (size_t)nw * 16 * (LA_BN + LA_PAD));
   int dev = 0;
   hipGetDevice(&dev);
   int lds_max = 0;
@@ -367,10 +377,11 @@ bool latent_attention_mfma(torch::Tensor out, torch::Tensor q_abs,
   const int64_t cus = prop->multiProcessorCount;
   const int64_t blocks = (int64_t)ntiles * hgroups;
   int nsplit = 1;
-  if (blocks < cus) {
+  const int64_t want_blocks = cus * (nw == 1 ? 4 : 1);
+  if (blocks < want_blocks) {
     const int64_t key_tiles = std::max<int64_t>(1, max_keys / LA_BN);
     nsplit = (int)std::min<int64_t>(
-        std::min<int64_t>(8, (cus + blocks - 1) / blocks),
+        std::min<int64_t>(8, (want_blocks + blocks - 1) / blocks),
         std::max<int64_t>(1, key_tiles / 4));
   }
   const bool pipe = blocks * nsplit < 2048;
@@ -388,15 +399,15 @@ bool latent_attention_mfma(torch::Tensor out, torch::Tensor q_abs,
       q_rot.stride(1) % 8 == 0 &&
       reinterpret_cast<uintptr_t>(q_abs.data_ptr()) % 16 == 0 &&
       reinterpret_cast<uintptr_t>(q_rot.data_ptr()) % 16 == 0;
-#define LAUNCH_LA2(KSV, NTV, PIPEV)                                           \
+#define LAUNCH_LA2(KSV, NTV, PIPEV, NWV)                                      \
   do {                                                                        \
-    auto kern = latent_attention_mfma_kernel<KSV, NTV, PIPEV>;                \
+    auto kern = latent_attention_mfma_kernel<KSV, NTV, PIPEV, NWV>;           \
     if (shmem > 64 * 1024)                                                    \
       (void)hipFuncSetAttribute((const void*)kern,                            \
                                 hipFuncAttributeMaxDynamicSharedMemorySize,   \
                                 (int)shmem);                                  \
     hipLaunchKernelGGL(                                                       \
-        kern, grid, dim3(256), shmem, stream, (uint16_t*)out.data_ptr(),      \
+        kern, grid, dim3(NWV * 64), shmem, stream, (uint16_t*)out.data_ptr(), \
         nsplit > 1 ? (float*)part_o.data_ptr() : nullptr,                     \
         nsplit > 1 ? (float*)part_ml.data_ptr() : nullptr, nsplit, T,         \
         (const uint16_t*)q_abs.data_ptr(), (int64_t)q_abs.stride(0),          \
@@ -412,10 +423,15 @@ bool latent_attention_mfma(torch::Tensor out, torch::Tensor q_abs,
   } while (0)
 #define LAUNCH_LA(KSV, NTV)                                                   \
   do {                                                                        \
-    if (pipe) LAUNCH_LA2(KSV, NTV, true);                                     \
-    else LAUNCH_LA2(KSV, NTV, false);                                         \
+    if (pipe) LAUNCH_LA2(KSV, NTV, true, 4);                                  \
+    else LAUNCH_LA2(KSV, NTV, false, 4);                                      \
   } while (0)
-  if (ks_n <= 4 && nt_n <= 4) LAUNCH_LA(4, 4);
+  if (nw == 1) {
+    // single-wave workgroups always prefetch (they have nobody to overlap
+    // with); many more of them fit, so the split target is per wave slot
+    if (ks_n <= 4 && nt_n <= 4) LAUNCH_LA2(4, 4, true, 1);
+    else LAUNCH_LA2(10, 16, true, 1);
+  } else if (ks_n <= 4 && nt_n <= 4) LAUNCH_LA(4, 4);
   else if (ks_n <= 10 && nt_n <= 16) LAUNCH_LA(10, 16);
   else LAUNCH_LA(18, 32);
 #undef LAUNCH_LA
