@@ -225,21 +225,29 @@ __global__ __launch_bounds__(NW * 64, ((NW == 4 && KS <= 10) ? 2 : 1)) void late
         mx = fmaxf(mx, s);
       }
       const float mn = fmaxf(m_run[r4], group_reduce_max<16>(mx));
-      alpha[r4] = expf(m_run[r4] - mn);
+      alpha[r4] = __expf(m_run[r4] - mn);
       m_run[r4] = mn;
       float rowsum = 0.0f;
 #pragma unroll
       for (int nt = 0; nt < 2; ++nt) {
-        const float p = expf(acc_s[nt][r4] - mn);   // exp(-inf) = 0
+        // hardware exponential: the result is rounded to bf16 for the
+        // P.C product anyway, and this loop is VALU-bound; exp(-inf) = 0
+        const float p = __expf(acc_s[nt][r4] - mn);
         rowsum += p;
         pw_s[(crow0 + r4) * crs + nt * 16 + ccol] = f32_to_bf16(p);
       }
       l_run[r4] = l_run[r4] * alpha[r4] + group_reduce_sum<16>(rowsum);
     }
+    // the running maxima settle after the first tiles: skip the rescale
+    // of the whole accumulator when no row of this wave moved
+    const bool moved = alpha[0] != 1.0f || alpha[1] != 1.0f ||
+                       alpha[2] != 1.0f || alpha[3] != 1.0f;
+    if (__any(moved)) {
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) {
+      for (int nt = 0; nt < NT; ++nt) {
 #pragma unroll
-      for (int r4 = 0; r4 < 4; ++r4) acc_o[nt][r4] *= alpha[r4];
+        for (int r4 = 0; r4 < 4; ++r4) acc_o[nt][r4] *= alpha[r4];
+      }
     }
 
     // ---- O += P . C : one 32-key step per 16-wide output tile ----
