@@ -209,6 +209,170 @@ def fedatar_preset(name: str, width: int, vocab: int, pattern: str,
                          layers=layers)
 
 
+# ---------------------------------------------------------------------------
+# Mekevik: parallel-block decoder (mixer and feed-forward read the same
+# residual through two norms and are added together) whose mixer is
+# windowed SIGMOID attention: per-key logistic weights instead of a
+# softmax, a learned bias per (distance bucket, head), weights mixed
+# across heads, grouped key/value heads with their own value width,
+# optional blending of every layer's values with the first layer's, and a
+# sigmoid output gate.  Feed-forwards: a clamped gated unit or routed
+# SwiGLU experts chosen by a softmax router.
+# ---------------------------------------------------------------------------
+def distance_bucket(n: int, rows: int, far: float) -> int:
+    """Row of a distance-bias table for a key n tokens back: distances
+    below rows/2 have a row each; beyond that rows are spaced
+    logarithmically and the last one is reached at distance `far`."""
+    import math
+
+    half = rows // 2
+    if n < half:
+        return n
+    step = math.log(n / half) / math.log(far / half) * (rows - half)
+    return min(rows - 1, half + int(math.floor(step)))
+
+
+@dataclass
+class SigmoidAttentionSpec:
+    heads: int = 1
+    kv_heads: int = 1          # query head h reads kv head h // (H/G)
+    dim: int = 64              # query/key entries per head
+    vdim: int = 64             # value entries per head
+    scale: float = 0.0         # score multiplier; 0 => dim**-0.5
+    window: int = 0            # keys seen per query incl. itself; 0 = all
+    bias_rows: int = 32        # rows of the distance-bias table
+    bias_far: float = 128.0    # distance that reaches the last row
+    v_mix: bool = False        # blend values with the first such layer's
+
+    def __post_init__(self):
+        if not self.scale:
+            self.scale = float(self.dim) ** -0.5
+        if self.heads % self.kv_heads:
+            raise ValueError("heads must be a multiple of kv_heads")
+
+    def bias_distances(self) -> int:
+        """Distances that need their own entry when the bucket table is
+        expanded per distance: everything from `bias_far` on shares the
+        last row, and a window never looks further than itself."""
+        import math
+
+        n = int(math.ceil(self.bias_far)) + 1
+        n = max(n, self.bias_rows // 2 + 1)
+        return min(n, self.window) if self.window > 0 else n
+
+
+@dataclass
+class ClampedGLUSpec:
+    ff: int = 0
+    limit: float = 7.0         # gate clamped above, linear part both sides
+
+
+@dataclass
+class RoutedGLUSpec:
+    experts: int = 1
+    top: int = 1
+    expert_ff: int = 0
+    scale: float = 1.0         # multiplies the renormalised top-k weights
+
+
+@dataclass
+class MekevikConfig:
+    name: str
+    hidden_size: int
+    vocab_size: int
+    layers: list               # LayerSpec(type="attention", ...)
+    norm_eps: float = 1e-6
+    embed_scale: float = 1.0
+    logit_scale: float = 1.0
+    max_position: int = 1 << 20     # no position table anywhere
+    architecture: str = "Mekevik"
+
+    @property
+    def num_layers(self) -> int:
+        return len(self.layers)
+
+    @property
+    def is_moe(self) -> bool:
+        return any(isinstance(l.mlp, RoutedGLUSpec) for l in self.layers)
+
+    def kv_bytes_per_token(self, itemsize: int = 2) -> int:
+        return max(itemsize, sum(
+            l.mixer.kv_heads * (l.mixer.dim + l.mixer.vdim) * itemsize
+            for l in self.layers))
+
+    @staticmethod
+    def from_dict(cfg: dict, name: str = "mekevik",
+                  shapes: Optional[dict] = None) -> "MekevikConfig":
+        """Parse the design's config.json.  `shapes` (tensor name ->
+        shape, from the checkpoint header) gives the sizes the json
+        leaves to the tensors (rows of each distance-bias table)."""
+        shapes = shapes or {}
+        layers = []
+        for i, l in enumerate(cfg["layers"]):
+            m = l.get("mixer") or {}
+            if l["type"] != "attention":
+                raise ValueError(f"layer {i}: unknown mixer {l['type']!r}")
+            rel = shapes.get(f"l{i}.mix.rel")
+            mixer = SigmoidAttentionSpec(
+                heads=int(m["heads"]),
+                kv_heads=int(m.get("kv_heads") or m["heads"]),
+                dim=int(m["dim"]), vdim=int(m.get("vdim") or m["dim"]),
+                scale=float(m.get("scale") or 0.0),
+                window=int((m.get("mask") or {}).get("size") or 0),
+                bias_rows=int(rel[0]) if rel else int(
+                    m.get("bias_rows", 32)),
+                bias_far=float(m["bias_max"]),
+                v_mix=bool(m.get("v_mix")))
+            f = l.get("mlp")
+            if f is None:
+                mlp = None
+            elif f["kind"] == "dense":
+                mlp = ClampedGLUSpec(ff=int(f["ff"]),
+                                     limit=float(f["limit"]))
+            elif f["kind"] == "moe":
+                r = f["router"]
+                mlp = RoutedGLUSpec(experts=int(r["experts"]),
+                                    top=int(r["top"]),
+                                    expert_ff=int(f["expert"]["ff"]),
+                                    scale=float(r.get("scale", 1.0)))
+            else:
+                raise ValueError(f"layer {i}: unknown mlp {f['kind']!r}")
+            layers.append(LayerSpec(type="attention", mixer=mixer, mlp=mlp))
+        return MekevikConfig(
+            name=name, hidden_size=int(cfg["width"]),
+            vocab_size=int(cfg["vocab"]), layers=layers,
+            norm_eps=float((cfg.get("norm") or {}).get("eps", 1e-6)),
+            embed_scale=float((cfg.get("embedding") or {}).get("scale",
+                                                               1.0)),
+            logit_scale=float(cfg.get("logit_scale", 1.0)))
+
+
+def mekevik_preset(name: str, width: int, vocab: int, pattern: str,
+                   heads: int, kv_heads: int, dim: int, vdim: int,
+                   window: int, ff: int, experts: int, top: int,
+                   expert_ff: int, bias_rows: int = 32,
+                   bias_far: float = 128.0, limit: float = 7.0,
+                   router_scale: float = 1.0, v_mix: bool = True,
+                   embed_scale: float = 1.0, logit_scale: float = 1.0
+                   ) -> MekevikConfig:
+    """Layer pattern string: one letter per layer for its feed-forward —
+    `d` (clamped dense unit), `m` (routed experts) or `-` (none)."""
+    layers = []
+    for tok in pattern.split():
+        mixer = SigmoidAttentionSpec(
+            heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim,
+            window=window, bias_rows=bias_rows, bias_far=bias_far,
+            v_mix=v_mix)
+        mlp = {"d": ClampedGLUSpec(ff=ff, limit=limit),
+               "m": RoutedGLUSpec(experts=experts, top=top,
+                                  expert_ff=expert_ff, scale=router_scale),
+               "-": None}[tok]
+        layers.append(LayerSpec(type="attention", mixer=mixer, mlp=mlp))
+    return MekevikConfig(name=name, hidden_size=width, vocab_size=vocab,
+                         layers=layers, embed_scale=embed_scale,
+                         logit_scale=logit_scale)
+
+
 # Architectures from the public model cards (random-init weights — no network).
 MODEL_PRESETS = {
     "llama-3-8b": ModelConfig(
@@ -346,6 +510,17 @@ MODEL_PRESETS = {
         heads=32, dim=128, rot_dim=64, vdim=128, kv_rank=512,
         q_rank=1536, window=4096, ff=14336, experts=8, top=2,
         expert_ff=14336, shared_ff=0, rot_base=1000000.0),
+    # tiny Mekevik for CPU tests / smoke: all three feed-forward kinds
+    "tiny-mekevik": mekevik_preset(
+        "tiny-mekevik", width=128, vocab=512, pattern="d m - m",
+        heads=4, kv_heads=2, dim=24, vdim=16, window=20, ff=192,
+        experts=6, top=2, expert_ff=48, bias_rows=12, bias_far=40.0,
+        limit=1.5, router_scale=1.5, embed_scale=0.5, logit_scale=0.5),
+    # layer-shape benchmark point at Mixtral-8x7B's width
+    "mekevik-4k": mekevik_preset(
+        "mekevik-4k", width=4096, vocab=32000, pattern="d m d m",
+        heads=32, kv_heads=8, dim=128, vdim=128, window=4096, ff=14336,
+        experts=8, top=2, expert_ff=14336, bias_rows=64, bias_far=4096.0),
     "tiny-moe": ModelConfig(
         name="tiny-moe",
         hidden_size=512,
@@ -460,6 +635,19 @@ class EngineConfig:
     def tiny_fedatar(**kw) -> "EngineConfig":
         defaults = dict(
             model=MODEL_PRESETS["tiny-fedatar"],
+            num_gpu_blocks=64,
+            max_num_seqs=8,
+            max_batched_tokens=2048,
+            max_model_len=512,
+            use_hip_graphs=False,
+        )
+        defaults.update(kw)
+        return EngineConfig(**defaults)
+
+    @staticmethod
+    def tiny_mekevik(**kw) -> "EngineConfig":
+        defaults = dict(
+            model=MODEL_PRESETS["tiny-mekevik"],
             num_gpu_blocks=64,
             max_num_seqs=8,
             max_batched_tokens=2048,

@@ -8,13 +8,15 @@ from pathlib import Path
 
 import torch
 
-from ..config import FedatarConfig, ModelConfig
+from ..config import FedatarConfig, MekevikConfig, ModelConfig
 
 
 def build_model(model_cfg, device, dtype):
     """Instantiate the model class for a config object."""
     if isinstance(model_cfg, FedatarConfig):
         from .fedatar import FedatarForCausalLM as cls
+    elif isinstance(model_cfg, MekevikConfig):
+        from .mekevik import MekevikForCausalLM as cls
     elif model_cfg.is_moe:
         from .mixtral import MixtralForCausalLM as cls
     else:
@@ -43,10 +45,14 @@ def safetensors_shapes(path: str) -> dict:
 
 
 def model_config_from_dir(path: str):
-    """Pick the architecture by the directory's config.json: the hybrid
-    design names itself with an `architecture` key; everything else is
-    read as a HuggingFace Llama-family config."""
+    """Pick the architecture by the directory's config.json: the
+    per-layer designs name themselves with an `architecture` key;
+    everything else is read as a HuggingFace Llama-family config."""
     cfg = json.loads((Path(path) / "config.json").read_text())
+    if cfg.get("architecture") == "Mekevik":
+        return MekevikConfig.from_dict(
+            cfg, name=Path(path).name or "mekevik",
+            shapes=safetensors_shapes(path))
     if cfg.get("architecture") == "Fedatar":
         return FedatarConfig.from_dict(
             cfg, name=Path(path).name or "fedatar",
@@ -65,4 +71,4 @@ def is_recurrent(model_cfg) -> bool:
 
 
 __all__ = ["build_model", "model_config_from_dir", "safetensors_shapes",
-           "is_recurrent", "ModelConfig", "FedatarConfig"]
+           "is_recurrent", "ModelConfig", "FedatarConfig", "MekevikConfig"]

@@ -4,6 +4,7 @@ A model describes what each layer keeps between steps; the engine
 allocates it once and passes layer i's buffer to layer i:
 
   ("paged_kv", heads, head_dim)  (K, V) pair [blocks, heads, block, dim]
+  ("paged_kv", heads, kdim, vdim)  the same with a value width of its own
   ("latent", width)              one paged row per token
                                  [blocks, block, width], compute dtype
   ("state", width)               one fp32 vector per SEQUENCE SLOT
@@ -60,9 +61,11 @@ def allocate_caches(specs: List[tuple], num_blocks: int, block_size: int,
     for spec in specs:
         kind = spec[0]
         if kind == "paged_kv":
-            shape = (num_blocks, spec[1], block_size, spec[2])
-            bufs.append((torch.zeros(shape, dtype=dtype, device=device),
-                         torch.zeros(shape, dtype=dtype, device=device)))
+            kshape = (num_blocks, spec[1], block_size, spec[2])
+            vshape = (num_blocks, spec[1], block_size,
+                      spec[3] if len(spec) > 3 else spec[2])
+            bufs.append((torch.zeros(kshape, dtype=dtype, device=device),
+                         torch.zeros(vshape, dtype=dtype, device=device)))
         elif kind == "latent":
             bufs.append(torch.zeros((num_blocks, block_size, spec[1]),
                                     dtype=dtype, device=device))

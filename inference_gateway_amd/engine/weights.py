@@ -335,6 +335,67 @@ def load_fedatar_weights(model, path: str) -> int:
     return n
 
 
+def load_mekevik_weights(model, path: str) -> int:
+    """Load a Mekevik checkpoint: tensors `embed`, `l<i>.norm1|norm2`,
+    `l<i>.mix.{q,k,v,g,o,q.norm,k.norm,rel,pb,talk,vmix}`,
+    `l<i>.mlp.{gate,up,down}` or `l<i>.mlp.router` and
+    `l<i>.mlp.e<j>.{gate,up,down}`, `final.norm`, `head`.  The engine's
+    fused layouts are assembled here: q|k|v|g stacked for the attention
+    input GEMM, gate|up stacked for the dense unit, experts stacked
+    K-major with gate|up side by side.  Norm weights, bias tables, the
+    head-mixing matrix and the router stay fp32; the per-distance bias
+    table is rebuilt from the loaded bucket table afterwards."""
+    from .config import ClampedGLUSpec, RoutedGLUSpec
+
+    sh = _Shards(path)
+    cfg = model.cfg
+    n = 0
+
+    def put(param, src, what):
+        nonlocal n
+        _copy(param, src, what)
+        n += 1
+
+    put(model.embed, sh.full("embed"), "embed")
+    for i, (spec, layer) in enumerate(zip(cfg.layers, model.layers)):
+        p = f"l{i}."
+        put(layer.norm1_w, sh.full(p + "norm1"), p + "norm1")
+        mx, m = layer.mixer, p + "mix."
+        put(mx.qkvg, torch.cat([sh.full(m + "q"), sh.full(m + "k"),
+                                sh.full(m + "v"), sh.full(m + "g")], 0),
+            m + "q|k|v|g")
+        put(mx.qnorm_w, sh.full(m + "q.norm"), m + "q.norm")
+        put(mx.knorm_w, sh.full(m + "k.norm"), m + "k.norm")
+        put(mx.rel, sh.full(m + "rel"), m + "rel")
+        put(mx.pb, sh.full(m + "pb"), m + "pb")
+        put(mx.talk, sh.full(m + "talk"), m + "talk")
+        put(mx.vmix, sh.full(m + "vmix").reshape(1), m + "vmix")
+        put(mx.o, sh.full(m + "o"), m + "o")
+        if spec.mlp is None:
+            continue
+        put(layer.norm2_w, sh.full(p + "norm2"), p + "norm2")
+        f, ff = layer.mlp, p + "mlp."
+        if isinstance(spec.mlp, ClampedGLUSpec):
+            put(f.gate_up, torch.cat([sh.full(ff + "gate"),
+                                      sh.full(ff + "up")], 0),
+                ff + "gate|up")
+            put(f.down, sh.full(ff + "down"), ff + "down")
+        elif isinstance(spec.mlp, RoutedGLUSpec):
+            put(f.router_w, sh.full(ff + "router"), ff + "router")
+            E = spec.mlp.experts
+            put(f.up_t, torch.stack([
+                torch.cat([sh.full(ff + f"e{e}.gate"),
+                           sh.full(ff + f"e{e}.up")], 0).t()
+                for e in range(E)]), ff + "e*.gate|up")
+            put(f.down_t, torch.stack(
+                [sh.full(ff + f"e{e}.down").t() for e in range(E)]),
+                ff + "e*.down")
+    put(model.final_norm_w, sh.full("final.norm"), "final.norm")
+    put(model.head, sh.full("head"), "head")
+    model.rebuild_tables()
+    return n
+
+
 def _is_gguf(path: str) -> bool:
     p = Path(path)
     if p.is_file():
@@ -356,6 +417,8 @@ def load_weights(model, path: str) -> int:
         return load_gguf_weights(model, path)
     if getattr(model.cfg, "architecture", "") == "Fedatar":
         return load_fedatar_weights(model, path)
+    if getattr(model.cfg, "architecture", "") == "Mekevik":
+        return load_mekevik_weights(model, path)
     if getattr(model.cfg, "is_moe", False):
         return load_mixtral_weights(model, path)
     return load_llama_weights(model, path)

@@ -437,8 +437,10 @@ def gate_heads(v, gate):
     return torch_ref.gate_heads_ref(v, gate)
 
 
-def moe_topk_route(logits, top_k: int, capacity: int = 0):
-    """logits [T, E] fp32 -> (softmax-over-chosen weights [T, K] fp32,
+def moe_topk_route(logits, top_k: int, capacity: int = 0,
+                   scale: float = 1.0):
+    """logits [T, E] fp32 -> (softmax-over-chosen weights [T, K] fp32
+    times `scale`,
     expert ids [T, K] int32, padded rows [T*K] int64 or None).  With
     capacity > 0 (>= T) the padded-dispatch row of every assignment,
     expert * capacity + rank, comes from the same launch.  Any K <= E <=
@@ -455,7 +457,111 @@ def moe_topk_route(logits, top_k: int, capacity: int = 0):
             dst = torch.empty(T * top_k, dtype=torch.int64,
                               device=logits.device)
             counts = torch.zeros(E, dtype=torch.int32, device=logits.device)
-        _hybrid.moe_topk_route(w, idx, logits, dst, counts, capacity)
+        _hybrid.moe_topk_route(w, idx, logits, dst, counts, capacity,
+                               scale)
         return w, idx, dst
     w, idx = torch_ref.moe_topk_route_ref(logits, top_k)
-    return w, idx, None
+    return (w * scale if scale != 1.0 else w), idx, None
+
+
+# ---------------------------------------------------------------------------
+# Parallel-block / sigmoid-attention mechanisms (same extension, same
+# typing rules: bf16 or fp32 activations, fp32 arithmetic).
+# ---------------------------------------------------------------------------
+GATED_ACT_SILU = torch_ref.GATED_ACT_SILU
+GATED_ACT_CLAMPED = torch_ref.GATED_ACT_CLAMPED
+
+
+def add_rmsnorm_pair(residual, delta_a, delta_b, w1, w2, eps: float,
+                     out_dtype):
+    """residual [T, D] fp32 += delta_a + delta_b (in place; either may
+    be None).  Returns (rmsnorm(residual) * w1, rmsnorm(residual) * w2)
+    from ONE pass and one statistic; w2 None gives (out, None)."""
+    if residual.is_cuda:
+        _require_hybrid()
+        out1 = torch.empty(residual.shape, dtype=out_dtype,
+                           device=residual.device)
+        out2 = None if w2 is None else torch.empty_like(out1)
+        _hybrid.add_rmsnorm_pair(out1, out2, residual, delta_a, delta_b,
+                                 w1, w2, eps)
+        return out1, out2
+    return torch_ref.add_rmsnorm_pair_ref(residual, delta_a, delta_b, w1,
+                                          w2, eps, out_dtype)
+
+
+def qk_norm_append(proj, slot_mapping, kcache, vcache, qnorm_w, knorm_w,
+                   v_first, lam: float, eps: float, heads: int,
+                   kv_heads: int, dim: int, vdim: int):
+    """Post-processing of a fused projection [T, H*dim | G*dim | G*vdim |
+    ...]: RMS norm over the whole query block and over the whole key
+    block, optional value blend (1-lam) v + lam v_first (v_first [T,
+    G*vdim], strided rows ok), keys and values appended to the paged
+    caches [blocks, G, block, d].  Returns the normed queries."""
+    if proj.is_cuda:
+        _require_hybrid()
+        q = torch.empty((proj.shape[0], heads * dim), dtype=proj.dtype,
+                        device=proj.device)
+        _hybrid.qk_norm_append(q, proj, slot_mapping, kcache, vcache,
+                               qnorm_w, knorm_w, v_first, lam, eps, heads,
+                               kv_heads, dim, vdim)
+        return q
+    return torch_ref.qk_norm_append_ref(
+        proj, slot_mapping, kcache, vcache, qnorm_w, knorm_w, v_first, lam,
+        eps, heads, kv_heads, dim, vdim)
+
+
+# bf16 batches run the MFMA tile kernel; off = the block-per-row kernel
+# (any dtype, any sizes) for everything
+SIGMOID_ATTENTION_MFMA = True
+
+
+def sigmoid_attention(q, kcache, vcache, block_table, row_seq, positions,
+                      dist_bias, talk, gate, scale: float, window: int,
+                      num_prefill_rows: int = 0, prefill_seq_lens=None):
+    """Windowed sigmoid attention over the paged cache with a bias per
+    (distance, head) (dist_bias [ND, H] fp32, distances from ND-1 on
+    share the last row), the heads' weights mixed by talk [H, H], grouped
+    key/value heads, and a sigmoid output gate (gate [T, H*vdim]
+    pre-activations, strided rows ok).  q [T, H*dim]; returns [T,
+    H*vdim].  Rows [0, num_prefill_rows) are prompt portions
+    (prefill_seq_lens = python row counts per sequence), the rest single
+    decoded tokens; every row reads its keys from the cache."""
+    if q.is_cuda:
+        _require_hybrid()
+        T = q.shape[0]
+        H = talk.shape[0]
+        out = torch.empty((T, H * vcache.shape[3]), dtype=q.dtype,
+                          device=q.device)
+        if q.dtype == torch.bfloat16 and SIGMOID_ATTENTION_MFMA and hasattr(
+                _hybrid, "sigmoid_attention_mfma"):
+            tq = _hybrid.sigmoid_attention_tile_rows()
+            tiles = _attention_tiles(
+                tq, num_prefill_rows,
+                tuple(prefill_seq_lens or ()) if num_prefill_rows else (),
+                T, q.device)
+            if _hybrid.sigmoid_attention_mfma(
+                    out, q, kcache, vcache, block_table, row_seq, positions,
+                    tiles[0], tiles[1], dist_bias, talk, gate, scale,
+                    window):
+                return out
+        _hybrid.sigmoid_attention(out, q, kcache, vcache, block_table,
+                                  row_seq, positions, dist_bias, talk, gate,
+                                  scale, window)
+        return out
+    return torch_ref.sigmoid_attention_ref(
+        q, kcache, vcache, block_table, row_seq, positions, dist_bias, talk,
+        gate, scale, window)
+
+
+def gated_act(gate_up, mode: int, limit: float = 0.0, alpha: float = 1.0):
+    """(gate | up) halves of the last dim -> one activation:
+    GATED_ACT_SILU silu(g) * u; GATED_ACT_CLAMPED with g' = min(g, limit),
+    u' = clamp(u, -limit, limit): g' * sigmoid(alpha g') * (u' + 1)."""
+    if gate_up.is_cuda:
+        _require_hybrid()
+        f = gate_up.shape[-1] // 2
+        out = torch.empty((*gate_up.shape[:-1], f), dtype=gate_up.dtype,
+                          device=gate_up.device)
+        _hybrid.gated_act(out, gate_up, mode, limit, alpha)
+        return out
+    return torch_ref.gated_act_ref(gate_up, mode, limit, alpha)

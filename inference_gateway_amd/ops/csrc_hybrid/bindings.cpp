@@ -21,7 +21,28 @@ void relu2(torch::Tensor out, torch::Tensor in);
 void gate_heads(torch::Tensor out, torch::Tensor v, torch::Tensor gate);
 void moe_topk_route(torch::Tensor weights, torch::Tensor idx,
                     torch::Tensor logits, c10::optional<torch::Tensor> dst,
-                    c10::optional<torch::Tensor> counts, int64_t capacity);
+                    c10::optional<torch::Tensor> counts, int64_t capacity,
+                    double scale);
+void add_rmsnorm_pair(torch::Tensor out1, c10::optional<torch::Tensor> out2,
+                      torch::Tensor residual,
+                      c10::optional<torch::Tensor> delta_a,
+                      c10::optional<torch::Tensor> delta_b, torch::Tensor w1,
+                      c10::optional<torch::Tensor> w2, double eps);
+void qk_norm_append(torch::Tensor q_out, torch::Tensor proj,
+                    torch::Tensor slot_mapping, torch::Tensor kcache,
+                    torch::Tensor vcache, torch::Tensor qnorm_w,
+                    torch::Tensor knorm_w,
+                    c10::optional<torch::Tensor> v_first, double lam,
+                    double eps, int64_t heads, int64_t kv_heads, int64_t dim,
+                    int64_t vdim);
+void gated_act(torch::Tensor out, torch::Tensor in, int64_t mode, double limit,
+               double alpha);
+void sigmoid_attention(torch::Tensor out, torch::Tensor q,
+                       torch::Tensor kcache, torch::Tensor vcache,
+                       torch::Tensor block_table, torch::Tensor row_seq,
+                       torch::Tensor positions, torch::Tensor dist_bias,
+                       torch::Tensor talk, torch::Tensor gate, double scale,
+                       int64_t window);
 void mingru_scan(torch::Tensor y, torch::Tensor zug, torch::Tensor state,
                  torch::Tensor seq_cu, torch::Tensor seq_start,
                  torch::Tensor seq_slots);
@@ -57,6 +78,14 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "[H,T,vd] values times [T,H] gates -> [T,H*vd]");
   m.def("moe_topk_route", &igw::moe_topk_route,
         "top-k experts and softmax over the chosen logits");
+  m.def("add_rmsnorm_pair", &igw::add_rmsnorm_pair,
+        "fp32 residual += two deltas; one RMS statistic, two weighted outputs");
+  m.def("qk_norm_append", &igw::qk_norm_append,
+        "whole-projection query/key RMS norms + value blend + paged append");
+  m.def("gated_act", &igw::gated_act,
+        "(gate | up) -> silu(g) u or the clamped gated unit");
+  m.def("sigmoid_attention", &igw::sigmoid_attention,
+        "windowed sigmoid attention, distance bias, head mixing, paged");
   m.def("mingru_scan", &igw::mingru_scan,
         "minGRU recurrence, one thread per (sequence, channel)");
   m.def("mingru_scan_chunked", &igw::mingru_scan_chunked,

@@ -8,7 +8,8 @@
 //                     every head
 //   xielu / relu2     feed-forward activations
 //   gate_heads        [H, T, vd] * gate[T, H] -> [T, H*vd]
-//   moe_topk_route    top-k experts + softmax over the chosen logits
+//   moe_topk_route    top-k experts + softmax over the chosen logits (times
+//                     a constant)
 //
 // One 256-thread block (4 waves) per token row for the row-wise kernels;
 // all arithmetic fp32, loads/stores in the activation type.
@@ -324,7 +325,8 @@ __global__ void moe_topk_route_kernel(float* __restrict__ weights,
                                       int64_t* __restrict__ dst,
                                       int32_t* __restrict__ counts,
                                       const float* __restrict__ logits, int T,
-                                      int E, int K, int capacity) {
+                                      int E, int K, int capacity,
+                                      float scale) {
   const int t = blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= T) return;
   const float* row = logits + (int64_t)t * E;
@@ -353,7 +355,7 @@ __global__ void moe_topk_route_kernel(float* __restrict__ weights,
     w[k] = e;
     z += e;
   }
-  for (int k = 0; k < K; ++k) w[k] = w[k] / z;
+  for (int k = 0; k < K; ++k) w[k] = w[k] / z * scale;
   // optional padded dispatch: row = expert * capacity + arrival rank (the
   // order inside an expert's segment carries no meaning: the gather back
   // uses the same rows)
@@ -368,7 +370,8 @@ __global__ void moe_topk_route_kernel(float* __restrict__ weights,
 
 void moe_topk_route(torch::Tensor weights, torch::Tensor idx,
                     torch::Tensor logits, c10::optional<torch::Tensor> dst,
-                    c10::optional<torch::Tensor> counts, int64_t capacity) {
+                    c10::optional<torch::Tensor> counts, int64_t capacity,
+                    double scale) {
   TORCH_CHECK(logits.is_cuda() && logits.dtype() == torch::kFloat32 &&
               logits.is_contiguous() && logits.dim() == 2);
   const int T = logits.size(0), E = logits.size(1), K = weights.size(1);
@@ -391,7 +394,8 @@ void moe_topk_route(torch::Tensor weights, torch::Tensor idx,
                      (int32_t*)idx.data_ptr(),
                      dst.has_value() ? (int64_t*)dst->data_ptr() : nullptr,
                      dst.has_value() ? (int32_t*)counts->data_ptr() : nullptr,
-                     (const float*)logits.data_ptr(), T, E, K, (int)capacity);
+                     (const float*)logits.data_ptr(), T, E, K, (int)capacity,
+                     (float)scale);
   HIP_CHECK_KERNEL();
 }
 

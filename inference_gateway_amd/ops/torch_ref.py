@@ -452,3 +452,104 @@ def rotary_inv_freq(base: float, dims: int, device="cpu"):
     rounded once to fp32 (the angle position * f_i is an fp32 product)."""
     i = torch.arange(dims // 2, dtype=torch.float64)
     return (float(base) ** (-2.0 * i / dims)).to(torch.float32).to(device)
+
+
+# ---------------------------------------------------------------------------
+# Parallel-block / sigmoid-attention mechanisms: one RMS statistic feeding
+# two norms, whole-projection query/key norm with value blending and paged
+# append, windowed sigmoid attention with a per-distance bias and mixing of
+# the weights across heads, gated feed-forward activations.  CPU
+# implementations behind ops.*; all arithmetic fp32.
+# ---------------------------------------------------------------------------
+def add_rmsnorm_pair_ref(residual, delta_a, delta_b, w1, w2, eps,
+                         out_dtype):
+    """residual (fp32, in place) += delta_a + delta_b (either may be
+    None); returns (x/rms(x) * w1, x/rms(x) * w2) — the second is None
+    when w2 is."""
+    if delta_a is not None and delta_b is not None:
+        residual.add_(delta_a.float() + delta_b.float())
+    elif delta_a is not None:
+        residual.add_(delta_a.float())
+    elif delta_b is not None:
+        residual.add_(delta_b.float())
+    n = residual * torch.rsqrt(
+        (residual * residual).mean(-1, keepdim=True) + eps)
+    return ((n * w1).to(out_dtype),
+            None if w2 is None else (n * w2).to(out_dtype))
+
+
+def qk_norm_append_ref(proj, slot_mapping, kcache, vcache, qnorm_w,
+                       knorm_w, v_first, lam, eps, H, G, dk, dv):
+    """proj [T, H*dk | G*dk | G*dv | ...]: RMS-norm the WHOLE query
+    block and the whole key block (one statistic each, over all heads),
+    blend the values with v_first (v <- (1-lam) v + lam v_first) when
+    given, append keys and values to the paged caches [blocks, G, block,
+    d]; returns the normed queries [T, H*dk]."""
+    T = proj.shape[0]
+    x = proj.float()
+    nq, nk, nv = H * dk, G * dk, G * dv
+    q = x[:, :nq]
+    q = q * torch.rsqrt((q * q).mean(-1, keepdim=True) + eps) * qnorm_w
+    k = x[:, nq:nq + nk]
+    k = k * torch.rsqrt((k * k).mean(-1, keepdim=True) + eps) * knorm_w
+    v = x[:, nq + nk:nq + nk + nv]
+    if v_first is not None:
+        v = (1.0 - lam) * v + lam * v_first.float()
+    bs = kcache.shape[2]
+    sm = slot_mapping.long()
+    blk, off = sm // bs, sm % bs
+    kcache[blk, :, off] = k.view(T, G, dk).to(kcache.dtype)
+    vcache[blk, :, off] = v.view(T, G, dv).to(vcache.dtype)
+    return q.to(proj.dtype)
+
+
+def sigmoid_attention_ref(q, kcache, vcache, block_table, row_seq,
+                          positions, dist_bias, talk, gate, scale, window):
+    """Row t (position p) of head g weighs key j, max(0, p-window+1) <= j
+    <= p, with sigmoid((q . k_j) * scale + dist_bias[min(p-j, last), g]);
+    head h then uses sum_g talk[h, g] * weight_g on the values of its own
+    key/value head.  The result, times sigmoid(gate), is [T, H*dv]."""
+    T = q.shape[0]
+    H = talk.shape[0]
+    G, bs, dk = kcache.shape[1], kcache.shape[2], kcache.shape[3]
+    dv = vcache.shape[3]
+    per = H // G
+    last = dist_bias.shape[0] - 1
+    out = torch.zeros((T, H, dv), dtype=torch.float32, device=q.device)
+    qf = q.float().view(T, G, per, dk)
+    pos = positions.tolist()
+    seqs = row_seq.tolist()
+    talk = talk.float()
+    for t in range(T):
+        p = pos[t]
+        lo = max(0, p - window + 1) if window > 0 else 0
+        j = torch.arange(lo, p + 1, device=q.device)
+        bt = block_table[seqs[t]].long()
+        blk, off = bt[j // bs], j % bs
+        kk = kcache[blk, :, off].float()                 # [n, G, dk]
+        vv = vcache[blk, :, off].float()                 # [n, G, dv]
+        sc = torch.einsum("gpd,ngd->gpn", qf[t], kk).reshape(H, -1) * scale
+        bias = dist_bias[torch.clamp(p - j, max=last)]   # [n, H]
+        w = torch.sigmoid(sc + bias.t())
+        mixed = (talk @ w).view(G, per, -1)
+        out[t] = torch.einsum("gpn,ngd->gpd", mixed, vv).reshape(H, dv)
+    out = out.view(T, H * dv) * torch.sigmoid(gate.float())
+    return out.to(q.dtype)
+
+
+GATED_ACT_SILU = 0       # silu(g) * u
+GATED_ACT_CLAMPED = 1    # min(g, L) * sigmoid(alpha * min(g, L))
+                         #   * (clamp(u, -L, L) + 1)
+
+
+def gated_act_ref(gate_up, mode, limit=0.0, alpha=1.0):
+    """gate_up [..., 2f] = (gate | up) -> [..., f]."""
+    f = gate_up.shape[-1] // 2
+    g, u = gate_up[..., :f].float(), gate_up[..., f:].float()
+    if mode == GATED_ACT_SILU:
+        y = g * torch.sigmoid(g) * u
+    else:
+        g = torch.clamp(g, max=limit)
+        u = torch.clamp(u, min=-limit, max=limit)
+        y = g * torch.sigmoid(alpha * g) * (u + 1.0)
+    return y.to(gate_up.dtype)
