@@ -84,6 +84,9 @@ def parse_args():
                          "equal layer sizes (engine prefill/decode "
                          "tokens/s and per-kernel roofline fractions); "
                          "prints its own JSON object")
+    ap.add_argument("--arch", type=str, default="fedatar",
+                    help="design for --arch-compare (fedatar | mekevik), "
+                         "each beside Mixtral")
     ap.add_argument("--arch-size", type=str, default="2k",
                     help="layer shape for --arch-compare (2k | 4k)")
     ap.add_argument("--num-gpu-blocks", type=int, default=0,
@@ -510,7 +513,10 @@ def main() -> None:
         return
     if args.arch_compare:
         sys.path.insert(0, str(Path(__file__).resolve().parent / "tools"))
-        import bench_hybrid
+        if args.arch == "mekevik":
+            import bench_parallel as bench_hybrid
+        else:
+            import bench_hybrid
 
         batch = args.batch if args.batch != 1024 else 64
         print(json.dumps(bench_hybrid.run(

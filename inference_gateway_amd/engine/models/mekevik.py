@@ -53,7 +53,7 @@ class SigmoidWindowAttention(nn.Module):
     per-distance table (`dist_bias`), so the kernel's inner loop does one
     indexed add."""
 
-    cache_kind = "paged_kv"
+    cache_kind = "paged_k_vt"
     GATE_ALPHA = 1.0
 
     def __init__(self, hidden: int, spec: SigmoidAttentionSpec, eps: float,
@@ -102,7 +102,7 @@ class SigmoidWindowAttention(nn.Module):
 
     def cache_spec(self) -> tuple:
         sp = self.spec
-        return ("paged_kv", sp.kv_heads, sp.dim, sp.vdim)
+        return ("paged_k_vt", sp.kv_heads, sp.dim, sp.vdim)
 
     def forward(self, h: torch.Tensor, fb: ForwardBatch, cache,
                 v_first: Optional[torch.Tensor]):
@@ -120,7 +120,7 @@ class SigmoidWindowAttention(nn.Module):
         o = ops.sigmoid_attention(
             q, kcache, vcache, fb.seq_block_table, fb.row_seq, fb.positions,
             self.dist_bias, self.talk, proj[:, v0 + self.nv:], sp.scale,
-            sp.window, fb.num_chunk_rows, fb.seq_lens)
+            sp.window, fb.num_chunk_rows, fb.seq_lens, fb.max_context)
         return F.linear(o, self.o), proj[:, v0:v0 + self.nv]
 
 

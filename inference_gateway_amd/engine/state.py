@@ -4,7 +4,12 @@ A model describes what each layer keeps between steps; the engine
 allocates it once and passes layer i's buffer to layer i:
 
   ("paged_kv", heads, head_dim)  (K, V) pair [blocks, heads, block, dim]
-  ("paged_kv", heads, kdim, vdim)  the same with a value width of its own
+  ("paged_k_vt", heads, kdim, vdim)  K [blocks, heads, block, kdim] and
+                                 V TRANSPOSED inside the page [blocks,
+                                 heads, vdim, block]: the keys of a page
+                                 are contiguous per value entry, which is
+                                 the operand layout of the P.V matrix
+                                 product (no transpose staging)
   ("latent", width)              one paged row per token
                                  [blocks, block, width], compute dtype
   ("state", width)               one fp32 vector per SEQUENCE SLOT
@@ -34,7 +39,7 @@ class LayerCaches(list):
         """Duplicate one page in every paged layer (forked sequences
         copy their partially filled tail page)."""
         for buf, spec in zip(self, self.specs):
-            if spec[0] == "paged_kv":
+            if spec[0] in ("paged_kv", "paged_k_vt"):
                 for t in buf:
                     t[dst].copy_(t[src])
             elif spec[0] == "latent":
@@ -61,9 +66,12 @@ def allocate_caches(specs: List[tuple], num_blocks: int, block_size: int,
     for spec in specs:
         kind = spec[0]
         if kind == "paged_kv":
+            shape = (num_blocks, spec[1], block_size, spec[2])
+            bufs.append((torch.zeros(shape, dtype=dtype, device=device),
+                         torch.zeros(shape, dtype=dtype, device=device)))
+        elif kind == "paged_k_vt":
             kshape = (num_blocks, spec[1], block_size, spec[2])
-            vshape = (num_blocks, spec[1], block_size,
-                      spec[3] if len(spec) > 3 else spec[2])
+            vshape = (num_blocks, spec[1], spec[3], block_size)
             bufs.append((torch.zeros(kshape, dtype=dtype, device=device),
                          torch.zeros(vshape, dtype=dtype, device=device)))
         elif kind == "latent":

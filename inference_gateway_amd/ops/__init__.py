@@ -496,7 +496,8 @@ def qk_norm_append(proj, slot_mapping, kcache, vcache, qnorm_w, knorm_w,
     ...]: RMS norm over the whole query block and over the whole key
     block, optional value blend (1-lam) v + lam v_first (v_first [T,
     G*vdim], strided rows ok), keys and values appended to the paged
-    caches [blocks, G, block, d].  Returns the normed queries."""
+    caches (keys [blocks, G, block, dim], values page-transposed
+    [blocks, G, vdim, block]).  Returns the normed queries."""
     if proj.is_cuda:
         _require_hybrid()
         q = torch.empty((proj.shape[0], heads * dim), dtype=proj.dtype,
@@ -517,7 +518,8 @@ SIGMOID_ATTENTION_MFMA = True
 
 def sigmoid_attention(q, kcache, vcache, block_table, row_seq, positions,
                       dist_bias, talk, gate, scale: float, window: int,
-                      num_prefill_rows: int = 0, prefill_seq_lens=None):
+                      num_prefill_rows: int = 0, prefill_seq_lens=None,
+                      max_context: int = 0):
     """Windowed sigmoid attention over the paged cache with a bias per
     (distance, head) (dist_bias [ND, H] fp32, distances from ND-1 on
     share the last row), the heads' weights mixed by talk [H, H], grouped
@@ -525,24 +527,27 @@ def sigmoid_attention(q, kcache, vcache, block_table, row_seq, positions,
     pre-activations, strided rows ok).  q [T, H*dim]; returns [T,
     H*vdim].  Rows [0, num_prefill_rows) are prompt portions
     (prefill_seq_lens = python row counts per sequence), the rest single
-    decoded tokens; every row reads its keys from the cache."""
+    decoded tokens; every row reads its keys from the cache.
+    max_context is a host hint (longest sequence in the batch) for
+    splitting keys over workgroups."""
     if q.is_cuda:
         _require_hybrid()
         T = q.shape[0]
         H = talk.shape[0]
-        out = torch.empty((T, H * vcache.shape[3]), dtype=q.dtype,
+        out = torch.empty((T, H * vcache.shape[2]), dtype=q.dtype,
                           device=q.device)
-        if q.dtype == torch.bfloat16 and SIGMOID_ATTENTION_MFMA and hasattr(
-                _hybrid, "sigmoid_attention_mfma"):
+        if q.dtype == torch.bfloat16 and SIGMOID_ATTENTION_MFMA:
             tq = _hybrid.sigmoid_attention_tile_rows()
             tiles = _attention_tiles(
                 tq, num_prefill_rows,
                 tuple(prefill_seq_lens or ()) if num_prefill_rows else (),
                 T, q.device)
+            ctx = max_context or 4096
+            max_keys = min(window, ctx) if window > 0 else ctx
             if _hybrid.sigmoid_attention_mfma(
                     out, q, kcache, vcache, block_table, row_seq, positions,
                     tiles[0], tiles[1], dist_bias, talk, gate, scale,
-                    window):
+                    window, max_keys):
                 return out
         _hybrid.sigmoid_attention(out, q, kcache, vcache, block_table,
                                   row_seq, positions, dist_bias, talk, gate,

@@ -63,6 +63,14 @@ bool latent_attention_mfma(torch::Tensor out, torch::Tensor q_abs,
                            torch::Tensor tile_nrows, torch::Tensor sink,
                            double scale, int64_t window, int64_t max_keys);
 int64_t latent_attention_tile_rows(int64_t H);
+bool sigmoid_attention_mfma(torch::Tensor out, torch::Tensor q,
+                            torch::Tensor kcache, torch::Tensor vcache,
+                            torch::Tensor block_table, torch::Tensor row_seq,
+                            torch::Tensor positions, torch::Tensor tile_row0,
+                            torch::Tensor tile_nrows, torch::Tensor dist_bias,
+                            torch::Tensor talk, torch::Tensor gate,
+                            double scale, int64_t window, int64_t max_keys);
+int64_t sigmoid_attention_tile_rows();
 }  // namespace igw
 
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
@@ -86,6 +94,11 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
         "(gate | up) -> silu(g) u or the clamped gated unit");
   m.def("sigmoid_attention", &igw::sigmoid_attention,
         "windowed sigmoid attention, distance bias, head mixing, paged");
+  m.def("sigmoid_attention_mfma", &igw::sigmoid_attention_mfma,
+        "windowed sigmoid attention on MFMA tiles (bf16); false = sizes do "
+        "not fit, use sigmoid_attention");
+  m.def("sigmoid_attention_tile_rows", &igw::sigmoid_attention_tile_rows,
+        "token rows per MFMA tile");
   m.def("mingru_scan", &igw::mingru_scan,
         "minGRU recurrence, one thread per (sequence, channel)");
   m.def("mingru_scan_chunked", &igw::mingru_scan_chunked,

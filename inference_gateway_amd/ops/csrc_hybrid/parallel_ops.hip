@@ -164,8 +164,9 @@ void add_rmsnorm_pair(torch::Tensor out1, c10::optional<torch::Tensor> out2,
 }
 
 // ---------------------------------------------------------------------------
-// proj row: [ q (H*dk) | k (G*dk) | v (G*dv) | ... ].  Caches are
-// [blocks, G, block, d]; slot = block * block_size + offset.
+// proj row: [ q (H*dk) | k (G*dk) | v (G*dv) | ... ].  Keys are cached as
+// [blocks, G, block, dk], values transposed inside the page as
+// [blocks, G, dv, block]; slot = block * block_size + offset.
 template <typename T>
 __global__ __launch_bounds__(PROW_BLOCK) void qk_norm_append_kernel(
     T* __restrict__ q_out, const T* __restrict__ proj, int64_t proj_stride,
@@ -203,7 +204,7 @@ __global__ __launch_bounds__(PROW_BLOCK) void qk_norm_append_kernel(
     const int g = d / DV, e = d % DV;
     float v = Act<T>::ld(x + NQ + NK + d);
     if (vf != nullptr) v = (1.0f - lam) * v + lam * Act<T>::ld(vf + d);
-    Act<T>::st(vcache + ((blk * G + g) * block_size + off) * DV + e, v);
+    Act<T>::st(vcache + ((blk * G + g) * DV + e) * block_size + off, v);
   }
 }
 
@@ -225,7 +226,7 @@ void qk_norm_append(torch::Tensor q_out, torch::Tensor proj,
               kcache.dtype() == proj.dtype());
   TORCH_CHECK(vcache.is_contiguous() && vcache.dim() == 4 &&
               vcache.size(0) == kcache.size(0) && vcache.size(1) == kv_heads &&
-              vcache.size(2) == kcache.size(2) && vcache.size(3) == vdim &&
+              vcache.size(3) == kcache.size(2) && vcache.size(2) == vdim &&
               vcache.dtype() == proj.dtype());
   TORCH_CHECK(slot_mapping.dtype() == torch::kInt32 &&
               slot_mapping.numel() == T);

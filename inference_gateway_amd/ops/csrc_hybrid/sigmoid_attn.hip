@@ -1,4 +1,6 @@
-// Windowed sigmoid attention over paged K/V caches (gfx950).
+// Windowed sigmoid attention over paged K/V caches (gfx950).  Keys are
+// cached as [blocks, G, block, dk]; values transposed inside the page,
+// [blocks, G, dv, block].
 //
 // For query row t (position p, sequence s), query head g (key/value head
 // c = g / (H/G)) and key j, max(0, p - window + 1) <= j <= p (window 0: from
@@ -91,9 +93,9 @@ __global__ __launch_bounds__(SA_BLOCK) void sigmoid_attention_rows_kernel(
         const int h = o / DV, d = o % DV, c = h / per;
         float a = acc[i];
         for (int jj = 0; jj < n; ++jj) {
-          const T* vr = vcache + (((int64_t)blk_lds[jj] * G + c) * block_size +
-                                  off_lds[jj]) * DV;
-          a += m_lds[h * SA_KT + jj] * Act<T>::ld(vr + d);
+          const T* vr = vcache + (((int64_t)blk_lds[jj] * G + c) * DV + d) *
+                                     block_size + off_lds[jj];
+          a += m_lds[h * SA_KT + jj] * Act<T>::ld(vr);
         }
         acc[i] = a;
       }
@@ -119,10 +121,10 @@ void sigmoid_attention_check(torch::Tensor out, torch::Tensor q,
   TORCH_CHECK(kcache.is_contiguous() && kcache.dim() == 4 &&
               vcache.is_contiguous() && vcache.dim() == 4);
   const int64_t T = q.size(0), H = talk.size(0), G = kcache.size(1);
-  const int64_t DK = kcache.size(3), DV = vcache.size(3);
+  const int64_t DK = kcache.size(3), DV = vcache.size(2);
   TORCH_CHECK(G >= 1 && H % G == 0 && q.size(1) == H * DK);
   TORCH_CHECK(vcache.size(0) == kcache.size(0) && vcache.size(1) == G &&
-              vcache.size(2) == kcache.size(2));
+              vcache.size(3) == kcache.size(2));
   TORCH_CHECK(kcache.dtype() == q.dtype() && vcache.dtype() == q.dtype());
   TORCH_CHECK(out.is_contiguous() && out.dtype() == q.dtype() &&
               out.dim() == 2 && out.size(0) == T && out.size(1) == H * DV);
@@ -146,7 +148,7 @@ void sigmoid_attention(torch::Tensor out, torch::Tensor q,
   sigmoid_attention_check(out, q, kcache, vcache, block_table, row_seq,
                           positions, dist_bias, talk, gate);
   const int T = q.size(0), H = talk.size(0), G = kcache.size(1);
-  const int DK = kcache.size(3), DV = vcache.size(3);
+  const int DK = kcache.size(3), DV = vcache.size(2);
   TORCH_CHECK(H * DV <= SA_BLOCK * 32,
               "sigmoid_attention: heads * vdim above 8192");
   const size_t shmem =

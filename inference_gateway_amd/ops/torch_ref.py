@@ -483,8 +483,9 @@ def qk_norm_append_ref(proj, slot_mapping, kcache, vcache, qnorm_w,
     """proj [T, H*dk | G*dk | G*dv | ...]: RMS-norm the WHOLE query
     block and the whole key block (one statistic each, over all heads),
     blend the values with v_first (v <- (1-lam) v + lam v_first) when
-    given, append keys and values to the paged caches [blocks, G, block,
-    d]; returns the normed queries [T, H*dk]."""
+    given, append keys to [blocks, G, block, dk] and values to the
+    page-transposed [blocks, G, dv, block]; returns the normed queries
+    [T, H*dk]."""
     T = proj.shape[0]
     x = proj.float()
     nq, nk, nv = H * dk, G * dk, G * dv
@@ -499,7 +500,7 @@ def qk_norm_append_ref(proj, slot_mapping, kcache, vcache, qnorm_w,
     sm = slot_mapping.long()
     blk, off = sm // bs, sm % bs
     kcache[blk, :, off] = k.view(T, G, dk).to(kcache.dtype)
-    vcache[blk, :, off] = v.view(T, G, dv).to(vcache.dtype)
+    vcache[blk, :, :, off] = v.view(T, G, dv).to(vcache.dtype)
     return q.to(proj.dtype)
 
 
@@ -512,7 +513,7 @@ def sigmoid_attention_ref(q, kcache, vcache, block_table, row_seq,
     T = q.shape[0]
     H = talk.shape[0]
     G, bs, dk = kcache.shape[1], kcache.shape[2], kcache.shape[3]
-    dv = vcache.shape[3]
+    dv = vcache.shape[2]            # values are [blocks, G, dv, block]
     per = H // G
     last = dist_bias.shape[0] - 1
     out = torch.zeros((T, H, dv), dtype=torch.float32, device=q.device)
@@ -527,7 +528,7 @@ def sigmoid_attention_ref(q, kcache, vcache, block_table, row_seq,
         bt = block_table[seqs[t]].long()
         blk, off = bt[j // bs], j % bs
         kk = kcache[blk, :, off].float()                 # [n, G, dk]
-        vv = vcache[blk, :, off].float()                 # [n, G, dv]
+        vv = vcache[blk, :, :, off].float()              # [n, G, dv]
         sc = torch.einsum("gpd,ngd->gpn", qf[t], kk).reshape(H, -1) * scale
         bias = dist_bias[torch.clamp(p - j, max=last)]   # [n, H]
         w = torch.sigmoid(sc + bias.t())

@@ -161,7 +161,7 @@ def test_qk_norm_append(device, H, G, dk, dv):
     for blend in (False, True):
         v_ref = ((1 - lam) * v_raw + lam * vf.to(F64)) if blend else v_raw
         kc = torch.zeros(nblocks, G, bs, dk, device=dev)
-        vc = torch.zeros(nblocks, G, bs, dv, device=dev)
+        vc = torch.zeros(nblocks, G, dv, bs, device=dev)
         q = ops.qk_norm_append(
             proj.to(dev), torch.tensor(slots, dtype=torch.int32, device=dev),
             kc, vc, wq.to(dev), wk.to(dev),
@@ -169,7 +169,7 @@ def test_qk_norm_append(device, H, G, dk, dv):
         assert torch.allclose(q.cpu().double(), q_ref, atol=3e-5)
         for t, s in enumerate(slots):
             kk = kc[s // bs, :, s % bs].reshape(-1).cpu().double()
-            vv = vc[s // bs, :, s % bs].reshape(-1).cpu().double()
+            vv = vc[s // bs, :, :, s % bs].reshape(-1).cpu().double()
             assert torch.allclose(kk, k_ref[t], atol=3e-5)
             assert torch.allclose(vv, v_ref[t], atol=3e-5)
         # nothing else was written
@@ -193,10 +193,10 @@ def _attention_case(H, G, dk, dv, T, bs, window, rows, far, seed, dev,
     talk = torch.eye(H) * 0.7 + torch.randn(H, H, generator=g) * 0.3
     pages, slots, nblocks = _paged_layout(T, bs, seed + 1)
     kc = torch.zeros(nblocks, G, bs, dk, dtype=dtype)
-    vc = torch.zeros(nblocks, G, bs, dv, dtype=dtype)
+    vc = torch.zeros(nblocks, G, dv, bs, dtype=dtype)
     for j, s in enumerate(slots):
         kc[s // bs, :, s % bs] = k[j]
-        vc[s // bs, :, s % bs] = v[j]
+        vc[s // bs, :, :, s % bs] = v[j]
     nd = int(math.ceil(far)) + 1
     nd = min(nd, window) if window else nd
     bias = torch.stack([rel[distance_bucket(n, rows, far)] + pb
@@ -299,7 +299,7 @@ def test_sigmoid_attention_far_key_window_and_page_edges(device, dtype,
         slot_row = a["block_table"][1, target // bs].item()
         a["kcache"][slot_row, :, target % bs] = kd.to(dt).to(dev)
         talk = a["talk"].double().cpu()
-        v_t = a["vcache"][slot_row, :, target % bs].double().cpu()  # [G,dv]
+        v_t = a["vcache"][slot_row, :, :, target % bs].double().cpu()
         per = H // G
         want = torch.stack([talk[h].sum() * v_t[h // per] for h in range(H)])
         want = want.reshape(-1) * oracle.logistic(
@@ -685,3 +685,105 @@ def test_trace_runner_command(tmp_path):
     assert not (out / "2.f32").exists()
     s3 = torch.from_numpy(np.fromfile(out / "3.f32", "<f4").reshape(-1, V))
     close(s3, ra[20:21], 2e-5)
+
+
+# ---------------------------------------------------------------------------
+# the bf16 matrix-core attention kernel (GPU only; pages of 8 or 16)
+# ---------------------------------------------------------------------------
+@pytest.mark.gpu
+@pytest.mark.parametrize("H,G,dk,dv,window,bs,T", [
+    (4, 2, 16, 16, 9, 8, 70),        # one head per wave, waves idle
+    (8, 4, 40, 24, 37, 16, 150),     # dk not a multiple of 32
+    (6, 3, 24, 40, 0, 16, 100),      # no window, dv not a multiple of 16
+    (1, 1, 8, 8, 1, 8, 40),          # sees only itself
+    (16, 4, 64, 64, 33, 16, 120),    # two heads per wave
+    (32, 8, 128, 128, 50, 16, 90),   # four heads per wave, value split
+    (24, 24, 32, 96, 64, 16, 130),   # three heads per wave, kv = heads
+])
+def test_sigmoid_attention_mfma(H, G, dk, dv, window, bs, T):
+    """Prompt portions with a cached prefix, whole prompts and decoded
+    rows in ONE launch, against the plain model on the same bf16 inputs."""
+    dev = "cuda:0"
+    rows_tab, far = 12, 45
+    scale = 1.3 / math.sqrt(dk)
+    a, p = _attention_case(H, G, dk, dv, T, bs, window, rows_tab, far,
+                           3 * H + dk, dev, torch.bfloat16)
+    start = 21                       # portion = positions [21, T-4)
+    dec = [T - 4, T - 1, 5]          # decoded rows, any order
+    rows = list(range(start, T - 4)) + dec
+    idx = torch.tensor(rows, device=dev)
+    ref = _attention_plain(p, rows, window, far, scale)
+    got = ops.sigmoid_attention(
+        a["q"][idx], a["kcache"], a["vcache"], a["block_table"],
+        a["row_seq"][idx], a["positions"][idx], a["dist_bias"], a["talk"],
+        a["gate"][idx], scale, window, T - 4 - start, [T - 4 - start], T)
+    err = (got.double().cpu() - ref).pow(2).mean().sqrt() / \
+        ref.pow(2).mean().sqrt()
+    assert float(err) < 1.2e-2, float(err)
+    worst = (got.double().cpu() - ref).abs().max() / ref.abs().max()
+    assert float(worst) < 4e-2, float(worst)
+    # the same rows through the block-per-row kernel agree as well
+    ops.SIGMOID_ATTENTION_MFMA = False
+    try:
+        slow = ops.sigmoid_attention(
+            a["q"][idx], a["kcache"], a["vcache"], a["block_table"],
+            a["row_seq"][idx], a["positions"][idx], a["dist_bias"],
+            a["talk"], a["gate"][idx], scale, window)
+    finally:
+        ops.SIGMOID_ATTENTION_MFMA = True
+    err = (slow.double().cpu() - ref).pow(2).mean().sqrt() / \
+        ref.pow(2).mean().sqrt()
+    assert float(err) < 6e-3, float(err)
+
+
+@pytest.mark.gpu
+def test_sigmoid_attention_mfma_key_splits():
+    """Few rows and many keys: the keys are split over workgroups and
+    summed; a long prompt in one launch crosses many tiles."""
+    dev = "cuda:0"
+    H, G, dk, dv, bs, T = 8, 4, 32, 32, 16, 900
+    for window in (0, 700):
+        scale = 1.0 / math.sqrt(dk)
+        a, p = _attention_case(H, G, dk, dv, T, bs, window, 16, 300, 5, dev,
+                               torch.bfloat16)
+        a["dist_bias"] = a["dist_bias"] - 3.0   # keep 900-key sums small
+        p["pb"] = p["pb"] - 3.0
+        rows = [T - 1, 640, 31, 32]
+        idx = torch.tensor(rows, device=dev)
+        ref = _attention_plain(p, rows, window, 300, scale)
+        got = ops.sigmoid_attention(
+            a["q"][idx], a["kcache"], a["vcache"], a["block_table"],
+            a["row_seq"][idx], a["positions"][idx], a["dist_bias"],
+            a["talk"], a["gate"][idx], scale, window, 0, None, T)
+        err = (got.double().cpu() - ref).pow(2).mean().sqrt() / \
+            ref.pow(2).mean().sqrt()
+        assert float(err) < 1.2e-2, (window, float(err))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("block", [8, 16])
+def test_bfloat16_engine_on_matrix_cores(tmp_path, block):
+    """The bf16 engine with pages the matrix-core kernel accepts: whole
+    prompt, ragged portions, decoding and a mixed batch agree with the
+    plain model and with each other."""
+    cfg = oracle.make_config(pattern=("d", "-", "d"), dim=16, vdim=24,
+                             window=19)
+    W = oracle.make_weights(cfg, seed=31)
+    tokens = toks(75, cfg["vocab"], 32)
+    ref = oracle.forward(cfg, W, tokens)
+    eng = make_engine(tmp_path, cfg, W, "cuda", dtype="bfloat16",
+                      block=block, blocks=40)
+    close(replay_all(eng, tokens, [75]), ref, 4e-2)
+    close(replay_all(eng, tokens, [5, 2, 30, 1, 1, 17, 19]), ref, 4e-2)
+    close(replay_all(eng, tokens, [40] + [1] * 35), ref, 4e-2)
+    # two requests side by side: a portion next to single tokens
+    a, b = eng.open_stream(), eng.open_stream()
+    outs = []
+    eng.replay_step([(a, tokens[:30])], {})
+    for n in range(5):
+        outs.append(eng.replay_step(
+            [(b, tokens[9 * n:9 * n + 9]), (a, tokens[30 + n:31 + n])],
+            {a: [0]}))
+    close(torch.cat(outs), ref[30:35], 4e-2)
+    eng.close_stream(a)
+    eng.close_stream(b)
