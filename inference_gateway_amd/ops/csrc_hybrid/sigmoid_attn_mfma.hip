@@ -39,7 +39,10 @@ constexpr int SM_BN = 32;        // keys per tile
 constexpr int SM_NW = 8;         // waves per workgroup
 constexpr int SM_WS = 32 + 8;    // LDS row stride (bf16 elements)
 
-template <int HW, int NT, int KS>
+// UNI: all heads of a wave read one key/value head (heads per wave divides
+// heads per group).  The K/V prefetches are compiled in where the register
+// file has room for them next to the Q fragments and the accumulators.
+template <int HW, int NT, int KS, bool UNI>
 __global__ __launch_bounds__(SM_NW * 64) void sigmoid_attention_mfma_kernel(
     uint16_t* __restrict__ out, float* __restrict__ part, int nsplit, int T,
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ kcache,
@@ -118,46 +121,109 @@ __global__ __launch_bounds__(SM_NW * 64) void sigmoid_attention_mfma_kernel(
 
   __syncthreads();
 
+  // UNI: the wave's K and V fragments are loaded once per tile and shared
+  // by its heads; the V fragments are requested at the top of the tile
+  // (PFV) and the NEXT tile's K fragments right after the scores (PFK), so
+  // both loads fly during the barriers and the mixing.
+  constexpr int REG_QA = 4 * HW * KS + 4 * HW * NT;
+  constexpr bool PFK = UNI && (REG_QA + 8 * KS + 4 * NT <= 112);
+  constexpr bool PFV =
+      UNI && (REG_QA + 4 * NT <= 128) && !(HW == 4 && KS == 4);
+  const int g0 = wave * hw_n;
+  const bool wave_on = g0 < H;
+  const int c0 = wave_on ? g0 / per : 0;
+  short8v kfrag[PFK ? 2 : 1][KS];
+  auto load_k = [&](int jt, int nt, int slot) {
+    const int j = min(jt * SM_BN + nt * 16 + frag_m, hi_all);
+    const uint16_t* kr =
+        kcache + (((int64_t)bt[j / block_size] * G + c0) * block_size +
+                  j % block_size) * DK + frag_k8;
+#pragma unroll
+    for (int kk = 0; kk < KS; ++kk) {
+      short8v b = {0, 0, 0, 0, 0, 0, 0, 0};
+      if (wave_on && kk * 32 + frag_k8 < DK)
+        b = *reinterpret_cast<const short8v*>(kr + kk * 32);
+      kfrag[slot][kk] = b;
+    }
+  };
+  if (PFK && t_a <= t_b) {
+    load_k(t_a, 0, 0);
+    load_k(t_a, 1, PFK ? 1 : 0);
+  }
+
   for (int jt = t_a; jt <= t_b; ++jt) {
     const int j0 = jt * SM_BN;
+    const int jk = j0 + frag_k8;
+    const int64_t vbase =
+        (int64_t)bt[min(jk / block_size, last_page)] * G * DV * block_size +
+        jk % block_size;
+    short8v vfrag[PFV ? NT : 1];
+    if (PFV) {
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        const int d = d_base + nt * 16 + frag_m;
+        short8v b = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (wave_on && nt < nt_n && d < DV)
+          b = *reinterpret_cast<const short8v*>(
+              vcache + vbase + ((int64_t)c0 * DV + d) * block_size);
+        vfrag[PFV ? nt : 0] = b;
+      }
+    }
     // ---- scores and weights of the owned heads ----
-    // the lane's key of each 16-key half, clamped into the sequence for the
-    // ADDRESS only (keys past the rows' reach are masked below)
-    int64_t kbase[2];
+    auto emit = [&](int g, int nt, const float4v& sc) {
+      const int j = j0 + nt * 16 + ccol;
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        const int i = crow0 + r4;
+        const int dist = p0 + i - j;
+        float w = 0.0f;
+        if (i < nrows && dist >= 0 && (window <= 0 || dist < window))
+          w = sigmoid_fast(sc[r4] * scale +
+                           dist_bias[min(dist, ND - 1) * H + g]);
+        w_s[(i * SM_BN + nt * 16 + ccol) * SM_WS + g] = f32_to_bf16(w);
+      }
+    };
 #pragma unroll
     for (int nt = 0; nt < 2; ++nt) {
-      const int j = min(j0 + nt * 16 + frag_m, hi_all);
-      kbase[nt] = ((int64_t)bt[j / block_size] * G * block_size +
-                   j % block_size) * DK + frag_k8;
-    }
+      if (UNI) {
+        float4v sacc[HW];
 #pragma unroll
-    for (int hw = 0; hw < HW; ++hw) {
-      const int g = wave * hw_n + hw;
-      if (hw < hw_n && g < H) {
-        const int c = g / per;
-        const int64_t coff = (int64_t)c * block_size * DK;
+        for (int hw = 0; hw < HW; ++hw) sacc[hw] = {0.f, 0.f, 0.f, 0.f};
+        if (!PFK) load_k(jt, nt, 0);
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt) {
-          const uint16_t* kr = kcache + kbase[nt] + coff;
-          float4v s = {0.f, 0.f, 0.f, 0.f};
+        for (int kk = 0; kk < KS; ++kk)
 #pragma unroll
-          for (int kk = 0; kk < KS; ++kk) {
-            short8v b = {0, 0, 0, 0, 0, 0, 0, 0};
-            if (kk * 32 + frag_k8 < DK)
-              b = *reinterpret_cast<const short8v*>(kr + kk * 32);
-            s = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qfrag[hw][kk], b, s, 0,
-                                                        0, 0);
-          }
-          const int j = j0 + nt * 16 + ccol;
+          for (int hw = 0; hw < HW; ++hw)
+            if (hw < hw_n)
+              sacc[hw] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                  qfrag[hw][kk], kfrag[PFK ? nt : 0][kk], sacc[hw], 0, 0, 0);
+        if (PFK && jt < t_b) load_k(jt + 1, nt, PFK ? nt : 0);
 #pragma unroll
-          for (int r4 = 0; r4 < 4; ++r4) {
-            const int i = crow0 + r4;
-            const int dist = p0 + i - j;
-            float w = 0.0f;
-            if (i < nrows && dist >= 0 && (window <= 0 || dist < window))
-              w = sigmoid_fast(s[r4] * scale +
-                               dist_bias[min(dist, ND - 1) * H + g]);
-            w_s[(i * SM_BN + nt * 16 + ccol) * SM_WS + g] = f32_to_bf16(w);
+        for (int hw = 0; hw < HW; ++hw)
+          if (hw < hw_n && g0 + hw < H) emit(g0 + hw, nt, sacc[hw]);
+      } else {
+        // heads of a wave on different key/value heads (or no room for
+        // shared fragments): load per head; the lane's key is clamped into
+        // the sequence for the ADDRESS only
+        const int j = min(j0 + nt * 16 + frag_m, hi_all);
+        const int64_t kbase = ((int64_t)bt[j / block_size] * G * block_size +
+                               j % block_size) * DK + frag_k8;
+#pragma unroll
+        for (int hw = 0; hw < HW; ++hw) {
+          const int g = g0 + hw;
+          if (hw < hw_n && g < H) {
+            const uint16_t* kr =
+                kcache + kbase + (int64_t)(g / per) * block_size * DK;
+            float4v sc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int kk = 0; kk < KS; ++kk) {
+              short8v bq = {0, 0, 0, 0, 0, 0, 0, 0};
+              if (kk * 32 + frag_k8 < DK)
+                bq = *reinterpret_cast<const short8v*>(kr + kk * 32);
+              sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qfrag[hw][kk], bq,
+                                                           sc, 0, 0, 0);
+            }
+            emit(g, nt, sc);
           }
         }
       }
@@ -187,24 +253,24 @@ __global__ __launch_bounds__(SM_NW * 64) void sigmoid_attention_mfma_kernel(
     __syncthreads();
     // ---- O_h += M_h . V_c : B fragments are 8 consecutive keys of one
     //      value entry, contiguous in the page-transposed cache ----
-    const int jk = j0 + frag_k8;
-    const int page = min(jk / block_size, last_page);
-    const int64_t vbase =
-        (int64_t)bt[page] * G * DV * block_size + jk % block_size;
 #pragma unroll
     for (int hw = 0; hw < HW; ++hw) {
-      const int h = wave * hw_n + hw;
+      const int h = g0 + hw;
       if (hw < hw_n && h < H) {
         const int c = h / per;
         const short8v a = *reinterpret_cast<const short8v*>(
             m_s + (h * SM_TQ + frag_m) * SM_WS + frag_k8);
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt) {
-          const int d = d_base + nt * 16 + frag_m;
           short8v b = {0, 0, 0, 0, 0, 0, 0, 0};
-          if (nt < nt_n && d < DV)
-            b = *reinterpret_cast<const short8v*>(
-                vcache + vbase + ((int64_t)c * DV + d) * block_size);
+          if (PFV) {
+            b = vfrag[PFV ? nt : 0];
+          } else {
+            const int d = d_base + nt * 16 + frag_m;
+            if (nt < nt_n && d < DV)
+              b = *reinterpret_cast<const short8v*>(
+                  vcache + vbase + ((int64_t)c * DV + d) * block_size);
+          }
           acc[hw][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
               a, b, acc[hw][nt], 0, 0, 0);
         }
@@ -285,13 +351,15 @@ bool sigmoid_attention_mfma(torch::Tensor out, torch::Tensor q,
   // shapes this kernel is built for; everything else takes the row kernel
   if (H > 4 * SM_NW || DK % 8 != 0 || DK > 128 || bs % 8 != 0) return false;
   const int hw_n = (H + SM_NW - 1) / SM_NW;           // heads per wave
+  // shared fragments need registers the largest tiles do not have left
+  const bool uni = (H / G) % hw_n == 0 && !(hw_n > 2 && DK > 64);
   const int nt_all = (DV + 15) / 16;
   // at most 16 accumulator tiles per wave: split the value width over
-  // gridDim.y beyond that
-  const int nt_max = std::min(4, 16 / hw_n);
+  // gridDim.y beyond that (which repeats the scores and the mixing)
+  const int nt_max = hw_n <= 2 ? 8 : 4;
   const int dsplit = (nt_all + nt_max - 1) / nt_max;
   const int nt_n = (nt_all + dsplit - 1) / dsplit;
-  if (nt_n > 4) return false;
+  if (nt_n > nt_max) return false;
   const size_t shmem =
       ((size_t)SM_TQ * SM_BN + (size_t)H * SM_TQ) * SM_WS * sizeof(uint16_t);
   if (T == 0 || ntiles == 0) return true;
@@ -310,16 +378,23 @@ bool sigmoid_attention_mfma(torch::Tensor out, torch::Tensor q,
     part = torch::empty({nsplit, T, (int64_t)H * DV},
                         q.options().dtype(torch::kFloat32));
 
-#define LAUNCH_SM(HWT, NTT, KST)                                              \
+#define LAUNCH_SM(HWT, NTT, KST)                       \
+  do {                                                 \
+    if (uni) LAUNCH_SM_U(HWT, NTT, KST, true);         \
+    else LAUNCH_SM_U(HWT, NTT, KST, false);            \
+  } while (0)
+#define LAUNCH_SM_U(HWT, NTT, KST, UNIT)                                      \
   do {                                                                        \
-    auto kern = sigmoid_attention_mfma_kernel<HWT, NTT, KST>;                 \
-    if (shmem > 48 * 1024) {                                                  \
+    auto kern = sigmoid_attention_mfma_kernel<HWT, NTT, KST, UNIT>;           \
+    static size_t lds_granted = 48 * 1024;                                    \
+    if (shmem > lds_granted) {                                                \
       if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),            \
                               hipFuncAttributeMaxDynamicSharedMemorySize,     \
                               (int)shmem) != hipSuccess) {                    \
         (void)hipGetLastError();                                              \
         return false;                                                         \
       }                                                                       \
+      lds_granted = shmem;                                                    \
     }                                                                         \
     hipLaunchKernelGGL(                                                       \
         kern, dim3(ntiles, dsplit, nsplit), dim3(SM_NW * 64), shmem, stream,  \
@@ -344,16 +419,19 @@ bool sigmoid_attention_mfma(torch::Tensor out, torch::Tensor q,
   } while (0)
   if (hw_n <= 1) {
     if (nt_n <= 2) LAUNCH_SM_KS(1, 2);
-    else LAUNCH_SM_KS(1, 4);
+    else if (nt_n <= 4) LAUNCH_SM_KS(1, 4);
+    else LAUNCH_SM_KS(1, 8);
   } else if (hw_n <= 2) {
     if (nt_n <= 2) LAUNCH_SM_KS(2, 2);
-    else LAUNCH_SM_KS(2, 4);
+    else if (nt_n <= 4) LAUNCH_SM_KS(2, 4);
+    else LAUNCH_SM_KS(2, 8);
   } else {
     if (nt_n <= 2) LAUNCH_SM_KS(4, 2);
     else LAUNCH_SM_KS(4, 4);
   }
 #undef LAUNCH_SM_KS
 #undef LAUNCH_SM
+#undef LAUNCH_SM_U
   HIP_CHECK_KERNEL();
   if (nsplit > 1) {
     const int64_t total = (int64_t)T * H * DV;

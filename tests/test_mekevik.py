@@ -787,3 +787,46 @@ def test_bfloat16_engine_on_matrix_cores(tmp_path, block):
     close(torch.cat(outs), ref[30:35], 4e-2)
     eng.close_stream(a)
     eng.close_stream(b)
+
+
+def test_local_provider_serves_a_checkpoint_directory(tmp_path):
+    """The gateway's local provider with LOCAL_MODEL=hf picks the
+    architecture from the directory's config.json and generates through
+    the async engine; the preset name works the same way."""
+    import asyncio
+
+    from inference_gateway_amd.config import LocalConfig
+    from inference_gateway_amd.providers.local import LocalProvider
+
+    cfg = oracle.make_config(vocab=300, pattern=("d", "m"))
+    W = oracle.make_weights(cfg, seed=35)
+    path = oracle.save_checkpoint(tmp_path / "m", cfg, W)
+    lc = LocalConfig(enabled=True, model="hf", max_num_seqs=4,
+                     max_model_len=128)
+    lc.num_gpu_blocks = 64
+    lc.weights_path = path
+    provider = LocalProvider(lc, device="cpu")
+    try:
+        assert isinstance(provider.engine.engine.cfg.model, MekevikConfig)
+
+        async def go():
+            return await provider.chat_completions({
+                "model": "local/hf",
+                "messages": [{"role": "user", "content": "hi"}],
+                "max_tokens": 3, "temperature": 0})
+
+        body = asyncio.run(go())
+        assert body["usage"]["completion_tokens"] == 3
+    finally:
+        provider.engine.shutdown()
+
+
+def test_preset_generates():
+    eng = LLMEngine(EngineConfig.tiny_mekevik(), device="cpu")
+    sid = eng.add_request(list(range(1, 30)),
+                          SamplingParams(max_new_tokens=5, temperature=0.0))
+    steps = 0
+    while not eng.is_finished() and steps < 50:
+        eng.step()
+        steps += 1
+    assert len(eng.get_output(sid).token_ids) == 5
