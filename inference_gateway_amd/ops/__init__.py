@@ -547,7 +547,7 @@ def sigmoid_attention(q, kcache, vcache, block_table, row_seq, positions,
             if _hybrid.sigmoid_attention_mfma(
                     out, q, kcache, vcache, block_table, row_seq, positions,
                     tiles[0], tiles[1], dist_bias, talk, gate, scale,
-                    window, max_keys):
+                    window, max_keys, num_prefill_rows):
                 return out
         _hybrid.sigmoid_attention(out, q, kcache, vcache, block_table,
                                   row_seq, positions, dist_bias, talk, gate,

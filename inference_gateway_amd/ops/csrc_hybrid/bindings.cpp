@@ -69,7 +69,8 @@ bool sigmoid_attention_mfma(torch::Tensor out, torch::Tensor q,
                             torch::Tensor positions, torch::Tensor tile_row0,
                             torch::Tensor tile_nrows, torch::Tensor dist_bias,
                             torch::Tensor talk, torch::Tensor gate,
-                            double scale, int64_t window, int64_t max_keys);
+                            double scale, int64_t window, int64_t max_keys,
+                            int64_t num_prefill_rows);
 int64_t sigmoid_attention_tile_rows();
 }  // namespace igw
 

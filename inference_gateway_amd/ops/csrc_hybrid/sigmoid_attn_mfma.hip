@@ -34,6 +34,11 @@ namespace igw {
 typedef __attribute__((ext_vector_type(8))) short short8v;
 typedef __attribute__((ext_vector_type(4))) float float4v;
 
+// round-to-nearest-even fp32 -> bf16 on the conversion unit
+DEVINLINE uint16_t sm_bf16(float f) {
+  return __builtin_bit_cast(uint16_t, (__bf16)f);
+}
+
 constexpr int SM_TQ = 16;        // query rows per workgroup
 constexpr int SM_BN = 32;        // keys per tile
 constexpr int SM_NW = 8;         // waves per workgroup
@@ -75,6 +80,8 @@ __global__ __launch_bounds__(SM_NW * 64) void sigmoid_attention_mfma_kernel(
   const int t_a = t_lo + (int)blockIdx.z * t_per;
   const int t_b = min(t_hi, t_a + t_per - 1);
   const int d_base = (int)blockIdx.y * nt_n * 16;   // first value entry here
+  // keys a row sees: 0 <= distance < wlim
+  const unsigned wlim = window > 0 ? (unsigned)window : 0x7fffffffu;
   const int last_page = hi_all / block_size;
 
   // head columns past H of the weight tile are never written: clear them
@@ -131,6 +138,7 @@ __global__ __launch_bounds__(SM_NW * 64) void sigmoid_attention_mfma_kernel(
       UNI && (REG_QA + 4 * NT <= 128) && !(HW == 4 && KS == 4);
   const int g0 = wave * hw_n;
   const bool wave_on = g0 < H;
+  const bool pair_ok = hw_n % 2 == 0 && per % 2 == 0;
   const int c0 = wave_on ? g0 / per : 0;
   short8v kfrag[PFK ? 2 : 1][KS];
   auto load_k = [&](int jt, int nt, int slot) {
@@ -170,17 +178,23 @@ __global__ __launch_bounds__(SM_NW * 64) void sigmoid_attention_mfma_kernel(
       }
     }
     // ---- scores and weights of the owned heads ----
+    // rows past the tile's last one are skipped as a whole (r4 >= nrows
+    // means every lane's row is): a decoded token pays for one row, not 16.
+    // Their LDS entries keep whatever they held — each query row only ever
+    // meets its own entries, and those rows are never stored.
     auto emit = [&](int g, int nt, const float4v& sc) {
-      const int j = j0 + nt * 16 + ccol;
+      const int dist0 = p0 + crow0 - (j0 + nt * 16 + ccol);
+      uint16_t* wp = w_s + ((crow0 * SM_BN) + nt * 16 + ccol) * SM_WS + g;
+      const float* bp = dist_bias + g;
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) {
-        const int i = crow0 + r4;
-        const int dist = p0 + i - j;
-        float w = 0.0f;
-        if (i < nrows && dist >= 0 && (window <= 0 || dist < window))
-          w = sigmoid_fast(sc[r4] * scale +
-                           dist_bias[min(dist, ND - 1) * H + g]);
-        w_s[(i * SM_BN + nt * 16 + ccol) * SM_WS + g] = f32_to_bf16(w);
+        if (r4 < nrows) {
+          const int dist = dist0 + r4;
+          float w = 0.0f;
+          if (crow0 + r4 < nrows && (unsigned)dist < wlim)
+            w = sigmoid_fast(sc[r4] * scale + bp[min(dist, ND - 1) * H]);
+          wp[r4 * SM_BN * SM_WS] = sm_bf16(w);
+        }
       }
     };
 #pragma unroll
@@ -208,22 +222,48 @@ __global__ __launch_bounds__(SM_NW * 64) void sigmoid_attention_mfma_kernel(
         const int j = min(j0 + nt * 16 + frag_m, hi_all);
         const int64_t kbase = ((int64_t)bt[j / block_size] * G * block_size +
                                j % block_size) * DK + frag_k8;
+        if (HW >= 2 && pair_ok) {
+          // two neighbouring heads of one key/value head share each K
+          // fragment
 #pragma unroll
-        for (int hw = 0; hw < HW; ++hw) {
-          const int g = g0 + hw;
-          if (hw < hw_n && g < H) {
-            const uint16_t* kr =
-                kcache + kbase + (int64_t)(g / per) * block_size * DK;
-            float4v sc = {0.f, 0.f, 0.f, 0.f};
+          for (int hw = 0; hw + 1 < HW; hw += 2) {
+            const int g = g0 + hw;
+            if (hw < hw_n && g < H) {
+              const uint16_t* kr =
+                  kcache + kbase + (int64_t)(g / per) * block_size * DK;
+              float4v s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int kk = 0; kk < KS; ++kk) {
-              short8v bq = {0, 0, 0, 0, 0, 0, 0, 0};
-              if (kk * 32 + frag_k8 < DK)
-                bq = *reinterpret_cast<const short8v*>(kr + kk * 32);
-              sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qfrag[hw][kk], bq,
-                                                           sc, 0, 0, 0);
+              for (int kk = 0; kk < KS; ++kk) {
+                short8v bq = {0, 0, 0, 0, 0, 0, 0, 0};
+                if (kk * 32 + frag_k8 < DK)
+                  bq = *reinterpret_cast<const short8v*>(kr + kk * 32);
+                s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qfrag[hw][kk], bq,
+                                                             s0, 0, 0, 0);
+                s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                    qfrag[hw + 1][kk], bq, s1, 0, 0, 0);
+              }
+              emit(g, nt, s0);
+              emit(g + 1, nt, s1);
             }
-            emit(g, nt, sc);
+          }
+        } else {
+#pragma unroll
+          for (int hw = 0; hw < HW; ++hw) {
+            const int g = g0 + hw;
+            if (hw < hw_n && g < H) {
+              const uint16_t* kr =
+                  kcache + kbase + (int64_t)(g / per) * block_size * DK;
+              float4v sc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+              for (int kk = 0; kk < KS; ++kk) {
+                short8v bq = {0, 0, 0, 0, 0, 0, 0, 0};
+                if (kk * 32 + frag_k8 < DK)
+                  bq = *reinterpret_cast<const short8v*>(kr + kk * 32);
+                sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(qfrag[hw][kk], bq,
+                                                             sc, 0, 0, 0);
+              }
+              emit(g, nt, sc);
+            }
           }
         }
       }
@@ -234,6 +274,7 @@ __global__ __launch_bounds__(SM_NW * 64) void sigmoid_attention_mfma_kernel(
     for (int q4 = 0; q4 < 4; ++q4) {
       const int nti = wave * 4 + q4;
       const int i = nti >> 1, jh = (nti & 1) * 16;
+      if (i >= nrows) continue;
       const short8v b = *reinterpret_cast<const short8v*>(
           w_s + (nti * 16 + frag_m) * SM_WS + frag_k8);
 #pragma unroll
@@ -245,7 +286,7 @@ __global__ __launch_bounds__(SM_NW * 64) void sigmoid_attention_mfma_kernel(
           for (int r4 = 0; r4 < 4; ++r4) {
             const int h = mt * 16 + crow0 + r4;
             if (h < H)
-              m_s[(h * SM_TQ + i) * SM_WS + jh + ccol] = f32_to_bf16(m[r4]);
+              m_s[(h * SM_TQ + i) * SM_WS + jh + ccol] = sm_bf16(m[r4]);
           }
         }
       }
@@ -253,26 +294,53 @@ __global__ __launch_bounds__(SM_NW * 64) void sigmoid_attention_mfma_kernel(
     __syncthreads();
     // ---- O_h += M_h . V_c : B fragments are 8 consecutive keys of one
     //      value entry, contiguous in the page-transposed cache ----
+    if (!PFV && HW >= 2 && REG_QA <= 96 && pair_ok) {
+      // two neighbouring heads of one key/value head share each V fragment
 #pragma unroll
-    for (int hw = 0; hw < HW; ++hw) {
-      const int h = g0 + hw;
-      if (hw < hw_n && h < H) {
-        const int c = h / per;
-        const short8v a = *reinterpret_cast<const short8v*>(
-            m_s + (h * SM_TQ + frag_m) * SM_WS + frag_k8);
+      for (int hw = 0; hw + 1 < HW; hw += 2) {
+        const int h = g0 + hw;
+        if (hw < hw_n && h < H) {
+          const int c = h / per;
+          const short8v a0 = *reinterpret_cast<const short8v*>(
+              m_s + (h * SM_TQ + frag_m) * SM_WS + frag_k8);
+          const short8v a1 = *reinterpret_cast<const short8v*>(
+              m_s + ((h + 1) * SM_TQ + frag_m) * SM_WS + frag_k8);
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-          short8v b = {0, 0, 0, 0, 0, 0, 0, 0};
-          if (PFV) {
-            b = vfrag[PFV ? nt : 0];
-          } else {
+          for (int nt = 0; nt < NT; ++nt) {
             const int d = d_base + nt * 16 + frag_m;
+            short8v bv = {0, 0, 0, 0, 0, 0, 0, 0};
             if (nt < nt_n && d < DV)
-              b = *reinterpret_cast<const short8v*>(
+              bv = *reinterpret_cast<const short8v*>(
                   vcache + vbase + ((int64_t)c * DV + d) * block_size);
+            acc[hw][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                a0, bv, acc[hw][nt], 0, 0, 0);
+            acc[hw + 1][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                a1, bv, acc[hw + 1][nt], 0, 0, 0);
           }
-          acc[hw][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-              a, b, acc[hw][nt], 0, 0, 0);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int hw = 0; hw < HW; ++hw) {
+        const int h = g0 + hw;
+        if (hw < hw_n && h < H) {
+          const int c = h / per;
+          const short8v a = *reinterpret_cast<const short8v*>(
+              m_s + (h * SM_TQ + frag_m) * SM_WS + frag_k8);
+#pragma unroll
+          for (int nt = 0; nt < NT; ++nt) {
+            short8v bv = {0, 0, 0, 0, 0, 0, 0, 0};
+            if (PFV) {
+              bv = vfrag[PFV ? nt : 0];
+            } else {
+              const int d = d_base + nt * 16 + frag_m;
+              if (nt < nt_n && d < DV)
+                bv = *reinterpret_cast<const short8v*>(
+                    vcache + vbase + ((int64_t)c * DV + d) * block_size);
+            }
+            acc[hw][nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                a, bv, acc[hw][nt], 0, 0, 0);
+          }
         }
       }
     }
@@ -308,14 +376,199 @@ __global__ __launch_bounds__(SM_NW * 64) void sigmoid_attention_mfma_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------
+// Single decoded rows: the matrix tiles are turned so that the M dimension
+// holds the HEADS of one key/value group instead of 16 query rows.  One
+// workgroup per (row, key split); wave c owns key/value head c: one K
+// fragment set scores all heads of the group, one V fragment set serves
+// them all, nothing is loaded twice and the register tiles are small enough
+// for several workgroups per compute unit.  The head mixing in the middle is
+// the same matrix product, over 32 keys.  For at most 8 key/value heads of
+// at most 16 query heads each and value widths up to 128.
+template <int NT, int KS>
+__global__ __launch_bounds__(SM_NW * 64) void sigmoid_attention_decode_mfma_kernel(
+    uint16_t* __restrict__ out, float* __restrict__ part, int nsplit, int T,
+    int row_first, const uint16_t* __restrict__ q,
+    const uint16_t* __restrict__ kcache, const uint16_t* __restrict__ vcache,
+    const int32_t* __restrict__ block_table, int max_blocks,
+    const int32_t* __restrict__ row_seq, const int32_t* __restrict__ positions,
+    const float* __restrict__ dist_bias, int ND,
+    const float* __restrict__ talk, const uint16_t* __restrict__ gate,
+    int64_t gate_stride, float scale, int window, int H, int G, int DK, int DV,
+    int block_size) {
+  __shared__ __attribute__((aligned(16))) uint16_t w_s[SM_BN * SM_WS];
+  __shared__ __attribute__((aligned(16))) uint16_t m_s[(32 + 16) * SM_WS];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int frag_m = lane & 15, frag_k8 = (lane >> 4) * 8;
+  const int crow0 = (lane >> 4) * 4, ccol = lane & 15;
+  const int per = H / G;
+  const int t = row_first + blockIdx.x;
+  const int pos = positions[t];
+  const int32_t* bt = block_table + (int64_t)row_seq[t] * max_blocks;
+  const int lo_all = window > 0 ? max(0, pos - window + 1) : 0;
+  const unsigned wlim = window > 0 ? (unsigned)window : 0x7fffffffu;
+  const int t_lo = lo_all / SM_BN, t_hi = pos / SM_BN;
+  const int t_per = (t_hi - t_lo + nsplit) / nsplit;
+  const int t_a = t_lo + (int)blockIdx.z * t_per;
+  const int t_b = min(t_hi, t_a + t_per - 1);
+  const int last_page = pos / block_size;
+  const int c = wave;                    // this wave's key/value head
+  const bool wave_on = c < G;
+  const int nt_n = (DV + 15) / 16;
+  const int mt_n = (H + 15) / 16;
+
+  for (int i = tid; i < SM_BN * SM_WS; i += SM_NW * 64) w_s[i] = 0;
+  for (int i = tid; i < (32 + 16) * SM_WS; i += SM_NW * 64) m_s[i] = 0;
+
+  // Q fragments: row = head of the group
+  short8v qfrag[KS];
+#pragma unroll
+  for (int kk = 0; kk < KS; ++kk) {
+    short8v f = {0, 0, 0, 0, 0, 0, 0, 0};
+    const int d = kk * 32 + frag_k8;
+    if (wave_on && frag_m < per && d < DK)
+      f = *reinterpret_cast<const short8v*>(
+          q + ((int64_t)t * H + c * per + frag_m) * DK + d);
+    qfrag[kk] = f;
+  }
+  // mixing jobs: (key half, head tile) pairs on the first waves
+  const int mix_nt = wave & 1, mix_mt = wave >> 1;
+  short8v tfrag = {0, 0, 0, 0, 0, 0, 0, 0};
+  if (mix_mt < mt_n) {
+    const int h = mix_mt * 16 + frag_m;
+    if (h < H) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const int g = frag_k8 + e;
+        if (g < H) tfrag[e] = (short)f32_to_bf16(talk[h * H + g]);
+      }
+    }
+  }
+  float4v acc[NT];
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) acc[nt] = {0.f, 0.f, 0.f, 0.f};
+  short8v kfrag[2][KS];
+  auto load_k = [&](int jt) {
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+      const int j = min(jt * SM_BN + nt * 16 + frag_m, pos);
+      const uint16_t* kr =
+          kcache + (((int64_t)bt[j / block_size] * G + c) * block_size +
+                    j % block_size) * DK + frag_k8;
+#pragma unroll
+      for (int kk = 0; kk < KS; ++kk) {
+        short8v b = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (wave_on && kk * 32 + frag_k8 < DK)
+          b = *reinterpret_cast<const short8v*>(kr + kk * 32);
+        kfrag[nt][kk] = b;
+      }
+    }
+  };
+  if (t_a <= t_b) load_k(t_a);
+  __syncthreads();
+
+  for (int jt = t_a; jt <= t_b; ++jt) {
+    const int j0 = jt * SM_BN;
+    const int jk = j0 + frag_k8;
+    short8v vfrag[NT];
+    {
+      const int64_t vbase =
+          ((int64_t)bt[min(jk / block_size, last_page)] * G + c) * DV *
+              block_size + jk % block_size;
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt) {
+        const int d = nt * 16 + frag_m;
+        short8v b = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (wave_on && nt < nt_n && d < DV)
+          b = *reinterpret_cast<const short8v*>(vcache + vbase +
+                                                (int64_t)d * block_size);
+        vfrag[nt] = b;
+      }
+    }
+    float4v sacc[2];
+#pragma unroll
+    for (int nt = 0; nt < 2; ++nt) {
+      sacc[nt] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int kk = 0; kk < KS; ++kk)
+        sacc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+            qfrag[kk], kfrag[nt][kk], sacc[nt], 0, 0, 0);
+    }
+    if (jt < t_b) load_k(jt + 1);
+    if (wave_on) {
+#pragma unroll
+      for (int nt = 0; nt < 2; ++nt) {
+        const int dist = pos - (j0 + nt * 16 + ccol);
+        const bool seen = (unsigned)dist < wlim;
+        const float* bp = dist_bias + min(max(dist, 0), ND - 1) * H + c * per;
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+          const int pp = crow0 + r4;
+          if (pp < per) {
+            float w = 0.0f;
+            if (seen) w = sigmoid_fast(sacc[nt][r4] * scale + bp[pp]);
+            w_s[(nt * 16 + ccol) * SM_WS + c * per + pp] = sm_bf16(w);
+          }
+        }
+      }
+    }
+    __syncthreads();
+    if (mix_mt < mt_n) {
+      const short8v b = *reinterpret_cast<const short8v*>(
+          w_s + (mix_nt * 16 + frag_m) * SM_WS + frag_k8);
+      float4v m = {0.f, 0.f, 0.f, 0.f};
+      m = __builtin_amdgcn_mfma_f32_16x16x32_bf16(tfrag, b, m, 0, 0, 0);
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        const int h = mix_mt * 16 + crow0 + r4;
+        if (h < H) m_s[h * SM_WS + mix_nt * 16 + ccol] = sm_bf16(m[r4]);
+      }
+    }
+    __syncthreads();
+    if (wave_on) {
+      // rows past the group's heads read other heads' (finite) entries or
+      // the zero tail; their results are never stored
+      const short8v a = *reinterpret_cast<const short8v*>(
+          m_s + (c * per + frag_m) * SM_WS + frag_k8);
+#pragma unroll
+      for (int nt = 0; nt < NT; ++nt)
+        if (nt < nt_n)
+          acc[nt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, vfrag[nt],
+                                                            acc[nt], 0, 0, 0);
+    }
+  }
+
+  if (!wave_on) return;
+  const int64_t HD = (int64_t)H * DV;
+#pragma unroll
+  for (int nt = 0; nt < NT; ++nt) {
+    const int d = nt * 16 + ccol;
+    if (nt >= nt_n || d >= DV) continue;
+#pragma unroll
+    for (int r4 = 0; r4 < 4; ++r4) {
+      const int pp = crow0 + r4;
+      if (pp >= per) continue;
+      const int64_t col = (int64_t)(c * per + pp) * DV + d;
+      if (nsplit == 1) {
+        const float gt = bf16_to_f32(gate[(int64_t)t * gate_stride + col]);
+        out[(int64_t)t * HD + col] =
+            f32_to_bf16(acc[nt][r4] * sigmoid_fast(gt));
+      } else {
+        part[((int64_t)blockIdx.z * T + t) * HD + col] = acc[nt][r4];
+      }
+    }
+  }
+}
+
 // out = sigmoid(gate) * sum over key splits
+// (rows [row_a, row_b) of T)
 __global__ void sigmoid_attention_merge_kernel(
     uint16_t* __restrict__ out, const float* __restrict__ part, int nsplit,
-    int64_t T, int64_t HD, const uint16_t* __restrict__ gate,
-    int64_t gate_stride) {
+    int64_t T, int64_t row_a, int64_t row_b, int64_t HD,
+    const uint16_t* __restrict__ gate, int64_t gate_stride) {
   const int64_t total = T * HD;
-  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
-       i += (int64_t)gridDim.x * blockDim.x) {
+  for (int64_t i = row_a * HD + (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+       i < row_b * HD; i += (int64_t)gridDim.x * blockDim.x) {
     float a = 0.0f;
     for (int z = 0; z < nsplit; ++z) a += part[z * total + i];
     const int64_t t = i / HD, c = i % HD;
@@ -337,17 +590,20 @@ bool sigmoid_attention_mfma(torch::Tensor out, torch::Tensor q,
                             torch::Tensor positions, torch::Tensor tile_row0,
                             torch::Tensor tile_nrows, torch::Tensor dist_bias,
                             torch::Tensor talk, torch::Tensor gate,
-                            double scale, int64_t window, int64_t max_keys) {
+                            double scale, int64_t window, int64_t max_keys,
+                            int64_t num_prefill_rows) {
   sigmoid_attention_check(out, q, kcache, vcache, block_table, row_seq,
                           positions, dist_bias, talk, gate);
   TORCH_CHECK(q.scalar_type() == torch::kBFloat16);
   const int T = q.size(0), H = talk.size(0), G = kcache.size(1);
   const int DK = kcache.size(3), DV = vcache.size(2);
   const int bs = kcache.size(2);
-  const int ntiles = tile_row0.numel();
+  const int ntiles_all = tile_row0.numel();
   TORCH_CHECK(tile_row0.dtype() == torch::kInt32 &&
               tile_nrows.dtype() == torch::kInt32 &&
-              tile_nrows.numel() == ntiles);
+              tile_nrows.numel() == ntiles_all);
+  TORCH_CHECK(num_prefill_rows >= 0 && num_prefill_rows <= T &&
+              T - num_prefill_rows <= ntiles_all);
   // shapes this kernel is built for; everything else takes the row kernel
   if (H > 4 * SM_NW || DK % 8 != 0 || DK > 128 || bs % 8 != 0) return false;
   const int hw_n = (H + SM_NW - 1) / SM_NW;           // heads per wave
@@ -362,22 +618,40 @@ bool sigmoid_attention_mfma(torch::Tensor out, torch::Tensor q,
   if (nt_n > nt_max) return false;
   const size_t shmem =
       ((size_t)SM_TQ * SM_BN + (size_t)H * SM_TQ) * SM_WS * sizeof(uint16_t);
-  if (T == 0 || ntiles == 0) return true;
+  if (T == 0 || ntiles_all == 0) return true;
   hipStream_t stream = at::cuda::getCurrentCUDAStream();
-
-  // key splits: fill the chip when there are few tiles (decode)
+  const int64_t HD = (int64_t)H * DV;
   const int key_tiles = std::max<int64_t>(1, (max_keys + SM_TQ) / SM_BN + 1);
-  int nsplit = 1;
-  if ((int64_t)ntiles * dsplit < 512)
-    nsplit = (int)std::min<int64_t>(
-        key_tiles, (512 + (int64_t)ntiles * dsplit - 1) /
-                       ((int64_t)ntiles * dsplit));
-  nsplit = std::max(1, std::min(nsplit, 64));
-  torch::Tensor part;
-  if (nsplit > 1)
-    part = torch::empty({nsplit, T, (int64_t)H * DV},
-                        q.options().dtype(torch::kFloat32));
+  auto splits_for = [&](int64_t groups, int64_t want) {
+    // key splits: fill the chip when there are few workgroups
+    int64_t n = 1;
+    if (groups < want) n = std::min<int64_t>(key_tiles, (want + groups - 1) / groups);
+    return (int)std::max<int64_t>(1, std::min<int64_t>(n, 64));
+  };
+  auto merge = [&](const torch::Tensor& part, int nsplit, int64_t ra,
+                   int64_t rb) {
+    const int64_t total = (rb - ra) * HD;
+    const int blocks = (int)std::min<int64_t>((total + 255) / 256, 8192);
+    hipLaunchKernelGGL(sigmoid_attention_merge_kernel, dim3(blocks), dim3(256),
+                       0, stream, (uint16_t*)out.data_ptr(),
+                       (const float*)part.data_ptr(), nsplit, (int64_t)T, ra,
+                       rb, HD, (const uint16_t*)gate.data_ptr(),
+                       (int64_t)gate.stride(0));
+  };
 
+  // single decoded rows go to the heads-as-rows kernel when its shape
+  // limits hold; prompt portions (and everything otherwise) to the
+  // rows-as-rows kernel
+  const int per = H / G;
+  const bool dec_ok = G <= SM_NW && per <= 16 && nt_all <= 8;
+  const int n_dec = dec_ok ? T - (int)num_prefill_rows : 0;
+  const int ntiles = ntiles_all - n_dec;
+
+  if (ntiles > 0) {
+    const int nsplit = splits_for((int64_t)ntiles * dsplit, 512);
+    torch::Tensor part;
+    if (nsplit > 1)
+      part = torch::empty({nsplit, T, HD}, q.options().dtype(torch::kFloat32));
 #define LAUNCH_SM(HWT, NTT, KST)                       \
   do {                                                 \
     if (uni) LAUNCH_SM_U(HWT, NTT, KST, true);         \
@@ -417,31 +691,64 @@ bool sigmoid_attention_mfma(torch::Tensor out, torch::Tensor q,
     if (DK <= 64) LAUNCH_SM(HWT, NTT, 2);     \
     else LAUNCH_SM(HWT, NTT, 4);              \
   } while (0)
-  if (hw_n <= 1) {
-    if (nt_n <= 2) LAUNCH_SM_KS(1, 2);
-    else if (nt_n <= 4) LAUNCH_SM_KS(1, 4);
-    else LAUNCH_SM_KS(1, 8);
-  } else if (hw_n <= 2) {
-    if (nt_n <= 2) LAUNCH_SM_KS(2, 2);
-    else if (nt_n <= 4) LAUNCH_SM_KS(2, 4);
-    else LAUNCH_SM_KS(2, 8);
-  } else {
-    if (nt_n <= 2) LAUNCH_SM_KS(4, 2);
-    else LAUNCH_SM_KS(4, 4);
-  }
+    if (hw_n <= 1) {
+      if (nt_n <= 2) LAUNCH_SM_KS(1, 2);
+      else if (nt_n <= 4) LAUNCH_SM_KS(1, 4);
+      else LAUNCH_SM_KS(1, 8);
+    } else if (hw_n <= 2) {
+      if (nt_n <= 2) LAUNCH_SM_KS(2, 2);
+      else if (nt_n <= 4) LAUNCH_SM_KS(2, 4);
+      else LAUNCH_SM_KS(2, 8);
+    } else {
+      if (nt_n <= 2) LAUNCH_SM_KS(4, 2);
+      else LAUNCH_SM_KS(4, 4);
+    }
 #undef LAUNCH_SM_KS
 #undef LAUNCH_SM
 #undef LAUNCH_SM_U
-  HIP_CHECK_KERNEL();
-  if (nsplit > 1) {
-    const int64_t total = (int64_t)T * H * DV;
-    const int blocks = (int)std::min<int64_t>((total + 255) / 256, 8192);
-    hipLaunchKernelGGL(sigmoid_attention_merge_kernel, dim3(blocks), dim3(256),
-                       0, stream, (uint16_t*)out.data_ptr(),
-                       (const float*)part.data_ptr(), nsplit, (int64_t)T,
-                       (int64_t)H * DV, (const uint16_t*)gate.data_ptr(),
-                       (int64_t)gate.stride(0));
     HIP_CHECK_KERNEL();
+    if (nsplit > 1) {
+      // rows of the launched tiles: [0, first decoded row) or all rows
+      merge(part, nsplit, 0, n_dec > 0 ? num_prefill_rows : (int64_t)T);
+      HIP_CHECK_KERNEL();
+    }
+  }
+
+  if (n_dec > 0) {
+    const int row_first = (int)num_prefill_rows;
+    const int nsplit = splits_for(n_dec, 1024);
+    torch::Tensor part;
+    if (nsplit > 1)
+      part = torch::empty({nsplit, T, HD}, q.options().dtype(torch::kFloat32));
+#define LAUNCH_DEC(NTT, KST)                                                  \
+  hipLaunchKernelGGL(                                                         \
+      (sigmoid_attention_decode_mfma_kernel<NTT, KST>), dim3(n_dec, 1, nsplit), \
+      dim3(SM_NW * 64), 0, stream, (uint16_t*)out.data_ptr(),                 \
+      nsplit > 1 ? (float*)part.data_ptr() : nullptr, nsplit, T, row_first,   \
+      (const uint16_t*)q.data_ptr(), (const uint16_t*)kcache.data_ptr(),      \
+      (const uint16_t*)vcache.data_ptr(),                                     \
+      (const int32_t*)block_table.data_ptr(), (int)block_table.size(1),       \
+      (const int32_t*)row_seq.data_ptr(),                                     \
+      (const int32_t*)positions.data_ptr(),                                   \
+      (const float*)dist_bias.data_ptr(), (int)dist_bias.size(0),             \
+      (const float*)talk.data_ptr(), (const uint16_t*)gate.data_ptr(),        \
+      (int64_t)gate.stride(0), (float)scale, (int)window, H, G, DK, DV, bs)
+    if (nt_all <= 2) {
+      if (DK <= 64) LAUNCH_DEC(2, 2);
+      else LAUNCH_DEC(2, 4);
+    } else if (nt_all <= 4) {
+      if (DK <= 64) LAUNCH_DEC(4, 2);
+      else LAUNCH_DEC(4, 4);
+    } else {
+      if (DK <= 64) LAUNCH_DEC(8, 2);
+      else LAUNCH_DEC(8, 4);
+    }
+#undef LAUNCH_DEC
+    HIP_CHECK_KERNEL();
+    if (nsplit > 1) {
+      merge(part, nsplit, row_first, T);
+      HIP_CHECK_KERNEL();
+    }
   }
   return true;
 }
