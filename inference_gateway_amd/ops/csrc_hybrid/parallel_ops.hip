@@ -167,7 +167,8 @@ void add_rmsnorm_pair(torch::Tensor out1, c10::optional<torch::Tensor> out2,
 // proj row: [ q (H*dk) | k (G*dk) | v (G*dv) | ... ].  Keys are cached as
 // [blocks, G, block, dk], values transposed inside the page as
 // [blocks, G, dv, block]; slot = block * block_size + offset.
-template <typename T>
+// VEC = 4: NQ, NK, DK % 4 == 0 and 16-byte aligned projection rows.
+template <typename T, int VEC>
 __global__ __launch_bounds__(PROW_BLOCK) void qk_norm_append_kernel(
     T* __restrict__ q_out, const T* __restrict__ proj, int64_t proj_stride,
     const int32_t* __restrict__ slot_mapping, T* __restrict__ kcache,
@@ -180,25 +181,55 @@ __global__ __launch_bounds__(PROW_BLOCK) void qk_norm_append_kernel(
   const T* x = proj + t * proj_stride;
   const int NK = G * DK, NV = G * DV;
   float sq = 0.0f, sk = 0.0f;
-  for (int d = threadIdx.x; d < NQ; d += PROW_BLOCK) {
-    const float v = Act<T>::ld(x + d);
-    sq += v * v;
-  }
-  for (int d = threadIdx.x; d < NK; d += PROW_BLOCK) {
-    const float v = Act<T>::ld(x + NQ + d);
-    sk += v * v;
+  if constexpr (VEC == 4) {
+    for (int d = threadIdx.x * 4; d < NQ; d += PROW_BLOCK * 4) {
+      const float4 v = Act4<T>::ld(x + d);
+      sq += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+    }
+    for (int d = threadIdx.x * 4; d < NK; d += PROW_BLOCK * 4) {
+      const float4 v = Act4<T>::ld(x + NQ + d);
+      sk += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+    }
+  } else {
+    for (int d = threadIdx.x; d < NQ; d += PROW_BLOCK) {
+      const float v = Act<T>::ld(x + d);
+      sq += v * v;
+    }
+    for (int d = threadIdx.x; d < NK; d += PROW_BLOCK) {
+      const float v = Act<T>::ld(x + NQ + d);
+      sk += v * v;
+    }
   }
   const float rq = 1.0f / sqrtf(prow_block_sum(sq, lds_a) / (float)NQ + eps);
   const float rk = 1.0f / sqrtf(prow_block_sum(sk, lds_b) / (float)NK + eps);
-  for (int d = threadIdx.x; d < NQ; d += PROW_BLOCK)
-    Act<T>::st(q_out + t * NQ + d, Act<T>::ld(x + d) * rq * wq[d]);
   const int slot = slot_mapping[t];
   const int64_t blk = slot / block_size, off = slot % block_size;
-  for (int d = threadIdx.x; d < NK; d += PROW_BLOCK) {
-    const int g = d / DK, e = d % DK;
-    Act<T>::st(kcache + ((blk * G + g) * block_size + off) * DK + e,
-               Act<T>::ld(x + NQ + d) * rk * wk[d]);
+  if constexpr (VEC == 4) {
+    for (int d = threadIdx.x * 4; d < NQ; d += PROW_BLOCK * 4) {
+      const float4 v = Act4<T>::ld(x + d);
+      const float4 g = *(const float4*)(wq + d);
+      Act4<T>::st(q_out + t * NQ + d,
+                  make_float4(v.x * rq * g.x, v.y * rq * g.y, v.z * rq * g.z,
+                              v.w * rq * g.w));
+    }
+    for (int d = threadIdx.x * 4; d < NK; d += PROW_BLOCK * 4) {
+      const int g = d / DK, e = d % DK;
+      const float4 v = Act4<T>::ld(x + NQ + d);
+      const float4 w = *(const float4*)(wk + d);
+      Act4<T>::st(kcache + ((blk * G + g) * block_size + off) * DK + e,
+                  make_float4(v.x * rk * w.x, v.y * rk * w.y, v.z * rk * w.z,
+                              v.w * rk * w.w));
+    }
+  } else {
+    for (int d = threadIdx.x; d < NQ; d += PROW_BLOCK)
+      Act<T>::st(q_out + t * NQ + d, Act<T>::ld(x + d) * rq * wq[d]);
+    for (int d = threadIdx.x; d < NK; d += PROW_BLOCK) {
+      const int g = d / DK, e = d % DK;
+      Act<T>::st(kcache + ((blk * G + g) * block_size + off) * DK + e,
+                 Act<T>::ld(x + NQ + d) * rk * wk[d]);
+    }
   }
+  // values go in transposed (one entry per page row): scalar stores
   const T* vf = v_first ? v_first + t * vf_stride : nullptr;
   for (int d = threadIdx.x; d < NV; d += PROW_BLOCK) {
     const int g = d / DV, e = d % DV;
@@ -239,18 +270,24 @@ void qk_norm_append(torch::Tensor q_out, torch::Tensor proj,
   }
   if (T == 0) return;
   hipStream_t stream = at::cuda::getCurrentCUDAStream();
+  const bool vec4 = NQ % 4 == 0 && dim % 4 == 0 && proj.stride(0) % 4 == 0 &&
+                    (uintptr_t)proj.data_ptr() % 16 == 0;
+#define LAUNCH_QKN(VEC)                                                       \
+  hipLaunchKernelGGL(                                                         \
+      (qk_norm_append_kernel<act_t, VEC>), dim3(T), dim3(PROW_BLOCK), 0,      \
+      stream, (act_t*)q_out.data_ptr(), (const act_t*)proj.data_ptr(),        \
+      (int64_t)proj.stride(0), (const int32_t*)slot_mapping.data_ptr(),       \
+      (act_t*)kcache.data_ptr(), (act_t*)vcache.data_ptr(),                   \
+      (const float*)qnorm_w.data_ptr(), (const float*)knorm_w.data_ptr(),     \
+      v_first.has_value() ? (const act_t*)v_first->data_ptr() : nullptr,      \
+      v_first.has_value() ? (int64_t)v_first->stride(0) : (int64_t)0,         \
+      (float)lam, (float)eps, NQ, (int)kv_heads, (int)dim, (int)vdim,         \
+      (int)kcache.size(2))
   IGW_DISPATCH_ACT(proj, {
-    hipLaunchKernelGGL(
-        (qk_norm_append_kernel<act_t>), dim3(T), dim3(PROW_BLOCK), 0, stream,
-        (act_t*)q_out.data_ptr(), (const act_t*)proj.data_ptr(),
-        (int64_t)proj.stride(0), (const int32_t*)slot_mapping.data_ptr(),
-        (act_t*)kcache.data_ptr(), (act_t*)vcache.data_ptr(),
-        (const float*)qnorm_w.data_ptr(), (const float*)knorm_w.data_ptr(),
-        v_first.has_value() ? (const act_t*)v_first->data_ptr() : nullptr,
-        v_first.has_value() ? (int64_t)v_first->stride(0) : (int64_t)0,
-        (float)lam, (float)eps, NQ, (int)kv_heads, (int)dim, (int)vdim,
-        (int)kcache.size(2));
+    if (vec4) LAUNCH_QKN(4);
+    else LAUNCH_QKN(1);
   });
+#undef LAUNCH_QKN
   HIP_CHECK_KERNEL();
 }
 

@@ -141,7 +141,8 @@ def _paged_layout(T, bs, seed, extra=3):
 
 @pytest.mark.parametrize("device", DEVICES)
 @pytest.mark.parametrize("H,G,dk,dv", [(4, 2, 12, 10), (1, 1, 5, 7),
-                                       (6, 6, 8, 8), (3, 1, 70, 33)])
+                                       (6, 6, 8, 8), (3, 1, 70, 33),
+                                       (4, 2, 16, 8)])
 def test_qk_norm_append(device, H, G, dk, dv):
     """Norm statistics span ALL heads of q (and of k); values are blended
     before they are paged; extra projection columns are left alone."""
@@ -149,7 +150,9 @@ def test_qk_norm_append(device, H, G, dk, dv):
     g = torch.Generator().manual_seed(H * 100 + dk)
     T, bs, eps, lam = 7, 4, 1e-4, 0.3125
     nq, nk, nv = H * dk, G * dk, G * dv
-    proj = torch.randn(T, nq + nk + nv + 5, generator=g) * 2
+    # the last case keeps rows 16-byte aligned (the vector path)
+    proj = torch.randn(T, nq + nk + nv + (4 if dk == 16 else 5),
+                       generator=g) * 2
     wq = torch.randn(nq, generator=g)
     wk = torch.randn(nk, generator=g)
     vf = torch.randn(T, nv + 3, generator=g)[:, 1:1 + nv]   # strided rows
