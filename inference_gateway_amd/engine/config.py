@@ -228,6 +228,10 @@ def distance_bucket(n: int, rows: int, far: float) -> int:
     half = rows // 2
     if n < half:
         return n
+    if half == 0 or far <= half:
+        # no logarithmic range to spread over: everything past the
+        # exact rows shares the last one
+        return rows - 1
     step = math.log(n / half) / math.log(far / half) * (rows - half)
     return min(rows - 1, half + int(math.floor(step)))
 
