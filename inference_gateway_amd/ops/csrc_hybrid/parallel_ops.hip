@@ -168,74 +168,124 @@ void add_rmsnorm_pair(torch::Tensor out1, c10::optional<torch::Tensor> out2,
 // [blocks, G, block, dk], values transposed inside the page as
 // [blocks, G, dv, block]; slot = block * block_size + offset.
 // VEC = 4: NQ, NK, DK % 4 == 0 and 16-byte aligned projection rows.
-template <typename T, int VEC>
+// R rows per block: with R = 8 the blended values of 8 consecutive batch
+// rows wait in LDS, and when those rows are 8 consecutive, 8-aligned slots
+// of one page (the usual case inside a prompt portion) each value entry's 8
+// tokens leave as ONE contiguous store into the page-transposed cache
+// instead of eight 2-byte stores 2 * block_size bytes apart.
+template <typename T>
+struct alignas(sizeof(T) * 8) Pack8 {
+  T v[8];
+};
+
+template <typename T, int VEC, int R>
 __global__ __launch_bounds__(PROW_BLOCK) void qk_norm_append_kernel(
     T* __restrict__ q_out, const T* __restrict__ proj, int64_t proj_stride,
     const int32_t* __restrict__ slot_mapping, T* __restrict__ kcache,
     T* __restrict__ vcache, const float* __restrict__ wq,
     const float* __restrict__ wk, const T* __restrict__ v_first,
     int64_t vf_stride, float lam, float eps, int NQ, int G, int DK, int DV,
-    int block_size) {
+    int block_size, int T_rows) {
   __shared__ float lds_a[PROW_BLOCK / 64], lds_b[PROW_BLOCK / 64];
-  const int64_t t = blockIdx.x;
-  const T* x = proj + t * proj_stride;
+  extern __shared__ __attribute__((aligned(16))) unsigned char qkn_smem[];
+  T* v_lds = reinterpret_cast<T*>(qkn_smem);          // [R][NV], R > 1 only
   const int NK = G * DK, NV = G * DV;
-  float sq = 0.0f, sk = 0.0f;
-  if constexpr (VEC == 4) {
-    for (int d = threadIdx.x * 4; d < NQ; d += PROW_BLOCK * 4) {
-      const float4 v = Act4<T>::ld(x + d);
-      sq += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+  const int64_t t0 = (int64_t)blockIdx.x * R;
+  const int nr = (int)min((int64_t)R, (int64_t)T_rows - t0);
+  for (int r = 0; r < nr; ++r) {
+    const int64_t t = t0 + r;
+    const T* x = proj + t * proj_stride;
+    float sq = 0.0f, sk = 0.0f;
+    if constexpr (VEC == 4) {
+      for (int d = threadIdx.x * 4; d < NQ; d += PROW_BLOCK * 4) {
+        const float4 v = Act4<T>::ld(x + d);
+        sq += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+      }
+      for (int d = threadIdx.x * 4; d < NK; d += PROW_BLOCK * 4) {
+        const float4 v = Act4<T>::ld(x + NQ + d);
+        sk += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+      }
+    } else {
+      for (int d = threadIdx.x; d < NQ; d += PROW_BLOCK) {
+        const float v = Act<T>::ld(x + d);
+        sq += v * v;
+      }
+      for (int d = threadIdx.x; d < NK; d += PROW_BLOCK) {
+        const float v = Act<T>::ld(x + NQ + d);
+        sk += v * v;
+      }
     }
-    for (int d = threadIdx.x * 4; d < NK; d += PROW_BLOCK * 4) {
-      const float4 v = Act4<T>::ld(x + NQ + d);
-      sk += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+    // (the two reductions use different LDS words, and each one's barrier
+    // separates the other's reads from its next writes)
+    const float rq = 1.0f / sqrtf(prow_block_sum(sq, lds_a) / (float)NQ + eps);
+    const float rk = 1.0f / sqrtf(prow_block_sum(sk, lds_b) / (float)NK + eps);
+    const int slot = slot_mapping[t];
+    const int64_t blk = slot / block_size, off = slot % block_size;
+    if constexpr (VEC == 4) {
+      for (int d = threadIdx.x * 4; d < NQ; d += PROW_BLOCK * 4) {
+        const float4 v = Act4<T>::ld(x + d);
+        const float4 g = *(const float4*)(wq + d);
+        Act4<T>::st(q_out + t * NQ + d,
+                    make_float4(v.x * rq * g.x, v.y * rq * g.y, v.z * rq * g.z,
+                                v.w * rq * g.w));
+      }
+      for (int d = threadIdx.x * 4; d < NK; d += PROW_BLOCK * 4) {
+        const int g = d / DK, e = d % DK;
+        const float4 v = Act4<T>::ld(x + NQ + d);
+        const float4 w = *(const float4*)(wk + d);
+        Act4<T>::st(kcache + ((blk * G + g) * block_size + off) * DK + e,
+                    make_float4(v.x * rk * w.x, v.y * rk * w.y, v.z * rk * w.z,
+                                v.w * rk * w.w));
+      }
+    } else {
+      for (int d = threadIdx.x; d < NQ; d += PROW_BLOCK)
+        Act<T>::st(q_out + t * NQ + d, Act<T>::ld(x + d) * rq * wq[d]);
+      for (int d = threadIdx.x; d < NK; d += PROW_BLOCK) {
+        const int g = d / DK, e = d % DK;
+        Act<T>::st(kcache + ((blk * G + g) * block_size + off) * DK + e,
+                   Act<T>::ld(x + NQ + d) * rk * wk[d]);
+      }
     }
-  } else {
-    for (int d = threadIdx.x; d < NQ; d += PROW_BLOCK) {
-      const float v = Act<T>::ld(x + d);
-      sq += v * v;
-    }
-    for (int d = threadIdx.x; d < NK; d += PROW_BLOCK) {
-      const float v = Act<T>::ld(x + NQ + d);
-      sk += v * v;
+    // values go in transposed (one entry per page row)
+    const T* vf = v_first ? v_first + t * vf_stride : nullptr;
+    for (int d = threadIdx.x; d < NV; d += PROW_BLOCK) {
+      float v = Act<T>::ld(x + NQ + NK + d);
+      if (vf != nullptr) v = (1.0f - lam) * v + lam * Act<T>::ld(vf + d);
+      if constexpr (R > 1) {
+        Act<T>::st(v_lds + r * NV + d, v);
+      } else {
+        const int g = d / DV, e = d % DV;
+        Act<T>::st(vcache + ((blk * G + g) * DV + e) * block_size + off, v);
+      }
     }
   }
-  const float rq = 1.0f / sqrtf(prow_block_sum(sq, lds_a) / (float)NQ + eps);
-  const float rk = 1.0f / sqrtf(prow_block_sum(sk, lds_b) / (float)NK + eps);
-  const int slot = slot_mapping[t];
-  const int64_t blk = slot / block_size, off = slot % block_size;
-  if constexpr (VEC == 4) {
-    for (int d = threadIdx.x * 4; d < NQ; d += PROW_BLOCK * 4) {
-      const float4 v = Act4<T>::ld(x + d);
-      const float4 g = *(const float4*)(wq + d);
-      Act4<T>::st(q_out + t * NQ + d,
-                  make_float4(v.x * rq * g.x, v.y * rq * g.y, v.z * rq * g.z,
-                              v.w * rq * g.w));
+  if constexpr (R > 1) {
+    __syncthreads();
+    const int s0 = slot_mapping[t0];
+    bool run = nr == R && block_size % R == 0 && (s0 % block_size) % R == 0;
+    for (int r = 1; r < nr; ++r)
+      run = run && slot_mapping[t0 + r] == s0 + r;
+    if (run) {
+      const int64_t blk = s0 / block_size, off = s0 % block_size;
+      for (int d = threadIdx.x; d < NV; d += PROW_BLOCK) {
+        const int g = d / DV, e = d % DV;
+        Pack8<T> p;
+#pragma unroll
+        for (int r = 0; r < 8; ++r) p.v[r] = v_lds[r * NV + d];
+        *reinterpret_cast<Pack8<T>*>(
+            vcache + ((blk * G + g) * DV + e) * block_size + off) = p;
+      }
+    } else {
+      for (int r = 0; r < nr; ++r) {
+        const int slot = slot_mapping[t0 + r];
+        const int64_t blk = slot / block_size, off = slot % block_size;
+        for (int d = threadIdx.x; d < NV; d += PROW_BLOCK) {
+          const int g = d / DV, e = d % DV;
+          vcache[((blk * G + g) * DV + e) * block_size + off] =
+              v_lds[r * NV + d];
+        }
+      }
     }
-    for (int d = threadIdx.x * 4; d < NK; d += PROW_BLOCK * 4) {
-      const int g = d / DK, e = d % DK;
-      const float4 v = Act4<T>::ld(x + NQ + d);
-      const float4 w = *(const float4*)(wk + d);
-      Act4<T>::st(kcache + ((blk * G + g) * block_size + off) * DK + e,
-                  make_float4(v.x * rk * w.x, v.y * rk * w.y, v.z * rk * w.z,
-                              v.w * rk * w.w));
-    }
-  } else {
-    for (int d = threadIdx.x; d < NQ; d += PROW_BLOCK)
-      Act<T>::st(q_out + t * NQ + d, Act<T>::ld(x + d) * rq * wq[d]);
-    for (int d = threadIdx.x; d < NK; d += PROW_BLOCK) {
-      const int g = d / DK, e = d % DK;
-      Act<T>::st(kcache + ((blk * G + g) * block_size + off) * DK + e,
-                 Act<T>::ld(x + NQ + d) * rk * wk[d]);
-    }
-  }
-  // values go in transposed (one entry per page row): scalar stores
-  const T* vf = v_first ? v_first + t * vf_stride : nullptr;
-  for (int d = threadIdx.x; d < NV; d += PROW_BLOCK) {
-    const int g = d / DV, e = d % DV;
-    float v = Act<T>::ld(x + NQ + NK + d);
-    if (vf != nullptr) v = (1.0f - lam) * v + lam * Act<T>::ld(vf + d);
-    Act<T>::st(vcache + ((blk * G + g) * DV + e) * block_size + off, v);
   }
 }
 
@@ -272,22 +322,34 @@ void qk_norm_append(torch::Tensor q_out, torch::Tensor proj,
   hipStream_t stream = at::cuda::getCurrentCUDAStream();
   const bool vec4 = NQ % 4 == 0 && dim % 4 == 0 && proj.stride(0) % 4 == 0 &&
                     (uintptr_t)proj.data_ptr() % 16 == 0;
-#define LAUNCH_QKN(VEC)                                                       \
+  // prompt-sized batches with wide values: 8 rows per block, values staged
+  // in LDS (measured: ahead from about 1024 value entries per token, where
+  // the scattered stores outweigh the rows' serialised reductions)
+  const size_t stage = (size_t)8 * NV * proj.element_size();
+  const bool rows8 = T >= 1024 && NV >= 1024 && stage <= 48 * 1024;
+#define LAUNCH_QKN(VEC)                                  \
+  do {                                                   \
+    if (rows8) LAUNCH_QKN_R(VEC, 8, (T + 7) / 8, stage); \
+    else LAUNCH_QKN_R(VEC, 1, T, 0);                     \
+  } while (0)
+#define LAUNCH_QKN_R(VEC, RR, BLOCKS, SHMEM)                                  \
   hipLaunchKernelGGL(                                                         \
-      (qk_norm_append_kernel<act_t, VEC>), dim3(T), dim3(PROW_BLOCK), 0,      \
-      stream, (act_t*)q_out.data_ptr(), (const act_t*)proj.data_ptr(),        \
+      (qk_norm_append_kernel<act_t, VEC, RR>), dim3(BLOCKS),                  \
+      dim3(PROW_BLOCK), SHMEM, stream, (act_t*)q_out.data_ptr(),              \
+      (const act_t*)proj.data_ptr(),                                          \
       (int64_t)proj.stride(0), (const int32_t*)slot_mapping.data_ptr(),       \
       (act_t*)kcache.data_ptr(), (act_t*)vcache.data_ptr(),                   \
       (const float*)qnorm_w.data_ptr(), (const float*)knorm_w.data_ptr(),     \
       v_first.has_value() ? (const act_t*)v_first->data_ptr() : nullptr,      \
       v_first.has_value() ? (int64_t)v_first->stride(0) : (int64_t)0,         \
       (float)lam, (float)eps, NQ, (int)kv_heads, (int)dim, (int)vdim,         \
-      (int)kcache.size(2))
+      (int)kcache.size(2), T)
   IGW_DISPATCH_ACT(proj, {
     if (vec4) LAUNCH_QKN(4);
     else LAUNCH_QKN(1);
   });
 #undef LAUNCH_QKN
+#undef LAUNCH_QKN_R
   HIP_CHECK_KERNEL();
 }
 

@@ -182,6 +182,55 @@ def test_qk_norm_append(device, H, G, dk, dv):
         assert float(flat[~written].abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("device", DEVICES)
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_qk_norm_append_many_rows(device, dtype):
+    """A prompt-sized batch: runs of consecutive slots that start on and
+    off 8-token boundaries, a run cut by the end of the batch, and
+    scattered slots, all land in the right place of the transposed
+    value pages."""
+    dev = _dev(device)
+    dt = getattr(torch, dtype)
+    g = torch.Generator().manual_seed(77)
+    H, G, dk, dv, bs, eps, lam = 8, 8, 16, 136, 16, 1e-5, 0.25
+    T = 1030
+    nq, nk, nv = H * dk, G * dk, G * dv     # nv wide enough for the
+    #                                         staged-store path on the GPU
+    proj = (torch.randn(T, nq + nk + nv + 8, generator=g) * 2).to(dt)
+    vf = torch.randn(T, nv, generator=g).to(dt)
+    wq = torch.randn(nq, generator=g)
+    wk = torch.randn(nk, generator=g)
+    nblocks = 200
+    slots = list(range(16, 16 + 600))                  # aligned run
+    slots += list(range(16 * 60 + 3, 16 * 60 + 3 + 200))   # off by three
+    free = torch.randperm(16 * 100, generator=g)[:T - 800] + 16 * 90
+    slots += free.tolist()                             # scattered
+    assert len(slots) == T and len(set(slots)) == T
+    P = proj.to(F64)
+    qn = P[:, :nq]
+    q_ref = qn / torch.sqrt((qn ** 2).mean(-1, keepdim=True) + eps) * wq
+    kn = P[:, nq:nq + nk]
+    k_ref = kn / torch.sqrt((kn ** 2).mean(-1, keepdim=True) + eps) * wk
+    v_ref = (1 - lam) * P[:, nq + nk:nq + nk + nv] + lam * vf.to(F64)
+    kc = torch.zeros(nblocks, G, bs, dk, device=dev, dtype=dt)
+    vc = torch.zeros(nblocks, G, dv, bs, device=dev, dtype=dt)
+    q = ops.qk_norm_append(
+        proj.to(dev), torch.tensor(slots, dtype=torch.int32, device=dev), kc,
+        vc, wq.to(dev), wk.to(dev), vf.to(dev), lam, eps, H, G, dk, dv)
+    tol = 3e-5 if dtype == "float32" else 4e-2
+    st = torch.tensor(slots)
+    got_k = kc.cpu()[st // bs, :, st % bs].reshape(T, nk).double()
+    got_v = vc.cpu()[st // bs, :, :, st % bs].reshape(T, nv).double()
+    assert float((q.cpu().double() - q_ref).abs().max()) < tol
+    assert float((got_k - k_ref).abs().max()) < tol
+    assert float((got_v - v_ref).abs().max()) < tol
+    # nothing else was written
+    mask = torch.ones(nblocks * bs, dtype=torch.bool)
+    mask[st] = False
+    flat = vc.cpu().permute(0, 3, 1, 2).reshape(nblocks * bs, -1)
+    assert float(flat[mask].abs().max()) == 0.0
+
+
 def _attention_case(H, G, dk, dv, T, bs, window, rows, far, seed, dev,
                     dtype=torch.float32):
     """Random q/k/v of one sequence, paged in shuffled order.  Returns the
