@@ -54,7 +54,6 @@ class SigmoidWindowAttention(nn.Module):
     indexed add."""
 
     cache_kind = "paged_k_vt"
-    GATE_ALPHA = 1.0
 
     def __init__(self, hidden: int, spec: SigmoidAttentionSpec, eps: float,
                  name: str, device, dtype):
